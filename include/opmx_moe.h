@@ -1,0 +1,130 @@
+/*
+ * opmx_moe.h - C ABI of libopmx_moe.so: the OPMX mixture-of-experts operators
+ * as hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer on the GPU that is current on the
+ *     calling thread; tensors are dense row-major; index tensors are int64,
+ *     exactly like the reference operators' outputs;
+ *   - `dtype` is an opmx_dtype value and applies to every floating tensor of
+ *     the call (the reference operators are single-dtype too);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     all work is enqueued on it, nothing synchronises the device;
+ *   - the library allocates nothing, frees nothing and keeps no pointer after
+ *     a call returns; scratch memory comes in through `workspace`;
+ *   - every function returns OPMX_OK (0) or a negative opmx_status; on error
+ *     nothing has been enqueued.  Faults inside a kernel surface, as with any
+ *     HIP work, at the next synchronisation.
+ *
+ * The reference (OpenPPL/ppl.pmx) has no native interface: its operators are
+ * torch.autograd.Function classes in torch_function/.  Each entry point below
+ * names the Python function whose eager branch it replaces.
+ */
+#ifndef OPMX_MOE_H_
+#define OPMX_MOE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OPMX_MOE_ABI_VERSION 1
+
+typedef enum opmx_dtype {
+    OPMX_DTYPE_F32 = 0,
+    OPMX_DTYPE_F16 = 1,
+    OPMX_DTYPE_BF16 = 2
+} opmx_dtype;
+
+typedef enum opmx_status {
+    OPMX_OK = 0,
+    OPMX_ERR_BAD_ARGUMENT = -1,   /* null pointer, negative size, k > E ...           */
+    OPMX_ERR_UNSUPPORTED = -2,    /* dtype / E / k outside what the kernels cover      */
+    OPMX_ERR_WORKSPACE = -3,      /* workspace missing or smaller than *_workspace_bytes */
+    OPMX_ERR_ALIGNMENT = -4,      /* a pointer or row pitch is not aligned as required */
+    OPMX_ERR_LAUNCH = -5          /* the HIP runtime refused a launch                  */
+} opmx_status;
+
+/* Epilogues of the grouped GEMM. */
+typedef enum opmx_epilogue {
+    OPMX_EPILOGUE_NONE = 0,
+    /* Y[r, i] = H[r, D+i] * H[r, i] * sigmoid(H[r, i]) with H = X W^T (+B) and
+     * D = N/2: SwiGLU (torch_function/SwiGLU.py:15-16, beta = 1) applied to the
+     * fp32 accumulators; Y is [R, N/2]. */
+    OPMX_EPILOGUE_SWIGLU = 1
+} opmx_epilogue;
+
+/* Limits of the routing kernels. */
+#define OPMX_MOE_MAX_EXPERTS 256
+#define OPMX_MOE_MAX_EXPERTS_PER_TOKEN 32
+
+int opmx_moe_abi_version(void);
+const char *opmx_status_string(int status);
+
+/* Router gate / plain linear.  Replaces Linear.forward,
+ * torch_function/Linear.py:25-33 (called from
+ * model_zoo/mixtral/modeling/dynamic_batching/Model.py:188):
+ *   Y[t, n] = sum_c X[t, c] * W[n, c] (+ B[n]),  fp32 accumulation.
+ * X [T,K], W [N,K], B [N] or NULL, Y [T,N]. */
+int opmx_linear(const void *X, const void *W, const void *B,
+                int64_t T, int64_t K, int64_t N, int dtype, void *Y, void *stream);
+
+/* MoeSelect.  Replaces MoeSelect.forward, torch_function/MoeSelect.py:37-64:
+ * top-k of scores ordered (value desc, expert id asc), softmax over the k
+ * picked values, stable sort of the T*k (token, slot) pairs by expert id.
+ *   X [T,H], scores [T,E]                                     (dtype)
+ *   X_expand_permute [T*k, H]                                 (dtype)
+ *   expert_weights [T,k]                                      (dtype)
+ *   invert_permutation [T*k] int64: row of X_expand_permute holding (t, slot)
+ *   expert_offset [E+1] int64: rows of expert e are [off[e], off[e+1])
+ * 1 <= k <= min(E, OPMX_MOE_MAX_EXPERTS_PER_TOKEN), E <= OPMX_MOE_MAX_EXPERTS.
+ * expert_ids may be NULL; otherwise it receives the picked ids [T,k] as int32
+ * (not an output of the reference operator; used by tests and fused callers). */
+size_t opmx_moe_select_workspace_bytes(int64_t T, int E, int k);
+int opmx_moe_select(const void *X, const void *scores, int64_t T, int64_t H, int E, int k,
+                    int dtype, void *X_expand_permute, void *expert_weights,
+                    int64_t *invert_permutation, int64_t *expert_offset, int32_t *expert_ids,
+                    void *workspace, size_t workspace_bytes, void *stream);
+
+/* Grouped expert GEMM.  Replaces the per-expert F.linear loops of
+ * MoeColumnParallelLinear.forward (torch_function/MoeColumnParallelLinear.py:58-69)
+ * and MoeRowParallelLinear.forward (torch_function/MoeRowParallelLinear.py:44-60)
+ * at tensor-parallel world size 1:
+ *   for e in [0,E), r in [off[e], off[e+1]):  Y[r,:] = X[r,:] W[e]^T (+ B[e])
+ * rows outside [off[0], off[E]) are set to zero.  expert_offset is read on the
+ * device; it must be non-decreasing with values in [0, R].
+ *   X [R,K], W [E,N,K], B [E,N] or NULL, Y [R,N] (or [R,N/2] with the SwiGLU epilogue).
+ * `rows_per_expert_hint` is the largest segment the caller can guarantee
+ * (for MoeSelect output: min(R, T)); 0 = unknown.  It only selects between
+ * kernel variants, never correctness. */
+size_t opmx_moe_grouped_gemm_workspace_bytes(int E, int64_t R, int64_t K, int64_t N, int dtype);
+int opmx_moe_column_parallel_linear(const void *X, const int64_t *expert_offset, const void *W,
+                                    const void *B, int E, int64_t R, int64_t K, int64_t N,
+                                    int dtype, int epilogue, int64_t rows_per_expert_hint,
+                                    void *Y, void *workspace, size_t workspace_bytes, void *stream);
+int opmx_moe_row_parallel_linear(const void *X, const int64_t *expert_offset, const void *W,
+                                 const void *B, int E, int64_t R, int64_t K, int64_t N,
+                                 int dtype, int64_t rows_per_expert_hint,
+                                 void *Y, void *workspace, size_t workspace_bytes, void *stream);
+
+/* SwiGLU.  Replaces SwiGLU.forward, torch_function/SwiGLU.py:11-17:
+ *   Y[r, i] = X[r, D+i] * X[r, i] * sigmoid(beta * X[r, i]);  X [R,2D], Y [R,D]. */
+int opmx_swiglu(const void *X, int64_t R, int64_t D, float beta, int dtype, void *Y, void *stream);
+
+/* Gated SiLU.  Replaces SiLU.forward, torch_function/SiLU.py:14-21:
+ *   Y[i] = gate[i] * X[i] * sigmoid(X[i])  (gate may be NULL);  n elements. */
+int opmx_silu(const void *X, const void *gate, int64_t n, int dtype, void *Y, void *stream);
+
+/* MoeReduce.  Replaces MoeReduce.forward, torch_function/MoeReduce.py:16-26:
+ *   out[t, :] = sum_{s<k} expert_weights[t,s] * Y[invert_permutation[t*k+s], :]
+ * summed in slot order in fp32, rounded once.  Y [T*k,N], out [T,N].
+ * invert_permutation values must lie in [0, T*k). */
+int opmx_moe_reduce(const void *Y, const void *expert_weights, const int64_t *invert_permutation,
+                    int64_t T, int k, int64_t N, int dtype, void *out, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OPMX_MOE_H_ */

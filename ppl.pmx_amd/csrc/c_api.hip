@@ -1,0 +1,199 @@
+// extern "C" surface of libopmx_moe.so: argument checks and kernel selection.
+// Declarations and the reference operator each entry point replaces are in
+// include/opmx_moe.h.
+#include <cstdlib>
+#include <cstring>
+
+#include "moe_gemm.h"
+
+using namespace opmx;
+
+namespace {
+
+inline bool dtype_ok(int d) { return d == OPMX_DTYPE_F32 || d == OPMX_DTYPE_F16 || d == OPMX_DTYPE_BF16; }
+inline size_t elt(int d) { return d == OPMX_DTYPE_F32 ? 4 : 2; }
+inline hipStream_t st(void *s) { return static_cast<hipStream_t>(s); }
+
+constexpr int64_t kStreamMaxRowsPerExpert = 128;
+
+int env_int(const char *name, int dflt)
+{
+    const char *v = std::getenv(name);
+    return (v && *v) ? std::atoi(v) : dflt;
+}
+
+// 0 = automatic, 1 = generic, 2 = tiled, 3 = stream  (tuning / test knob)
+int forced_kernel()
+{
+    const char *v = std::getenv("OPMX_MOE_GEMM");
+    if (!v || !*v) return 0;
+    if (!std::strcmp(v, "generic")) return 1;
+    if (!std::strcmp(v, "tiled")) return 2;
+    if (!std::strcmp(v, "stream")) return 3;
+    return 0;
+}
+
+}  // namespace
+
+namespace opmx {
+
+size_t grouped_gemm_workspace_bytes(int E, int64_t R, int64_t K, int64_t N, int dtype)
+{
+    (void)E;
+    (void)K;
+    // Only the streaming kernel with a fused epilogue stages [R,N] values.
+    if (R <= 0 || N <= 0 || R > kStreamMaxRowsPerExpert * OPMX_MOE_MAX_EXPERTS_PER_TOKEN) return 256;
+    return static_cast<size_t>(ceil_div(R * N * static_cast<int64_t>(elt(dtype)), 256) * 256);
+}
+
+int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
+                        int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint, void *Y, void *ws,
+                        size_t ws_bytes, hipStream_t s)
+{
+    const int64_t ncols = epilogue == OPMX_EPILOGUE_SWIGLU ? N / 2 : N;
+    if (R == 0 || ncols == 0) return OPMX_OK;
+    const bool lowp = dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16;
+    const bool mfma_ok = lowp && K > 0 && K % 8 == 0 && aligned16(X) && aligned16(W) &&
+                         N * K < (int64_t{1} << 31) && R * K < (int64_t{1} << 40);
+    const bool tiled_ok = mfma_ok && K % 64 == 0;
+    int64_t hint = rows_hint > 0 && rows_hint < R ? rows_hint : R;
+    const size_t stage = static_cast<size_t>(R * N) * elt(dtype);
+    const bool stream_ws = epilogue == OPMX_EPILOGUE_NONE || (ws && ws_bytes >= stage);
+    const int force = forced_kernel();
+
+    int choice;   // 1 generic, 2 tiled, 3 stream
+    if (force == 3 && mfma_ok && stream_ws) choice = 3;
+    else if (force == 2 && tiled_ok) choice = 2;
+    else if (force == 1) choice = 1;
+    else if (mfma_ok && stream_ws && hint <= kStreamMaxRowsPerExpert) choice = 3;
+    else if (tiled_ok) choice = 2;
+    else choice = 1;
+
+    if (choice == 3) {
+        const int variant = env_int("OPMX_MOE_GEMM_STREAM_VARIANT", 0);
+        if (epilogue == OPMX_EPILOGUE_NONE)
+            return launch_gemm_stream(X, off, W, B, E, R, K, N, dtype, epilogue, hint, variant, Y, s);
+        int rc = launch_gemm_stream(X, off, W, B, E, R, K, N, dtype, OPMX_EPILOGUE_NONE, hint, variant, ws, s);
+        if (rc != OPMX_OK) return rc;
+        return launch_swiglu(ws, R, N / 2, 1.0f, dtype, Y, s);
+    }
+    if (choice == 2)
+        return launch_gemm_tiled(X, off, W, B, E, R, K, N, dtype, epilogue,
+                                 env_int("OPMX_MOE_GEMM_TILED_VARIANT", 0), Y, s);
+    return launch_gemm_generic(X, off, W, B, E, R, K, N, dtype, epilogue, Y, s);
+}
+
+}  // namespace opmx
+
+extern "C" {
+
+int opmx_moe_abi_version(void) { return OPMX_MOE_ABI_VERSION; }
+
+const char *opmx_status_string(int status)
+{
+    switch (status) {
+        case OPMX_OK: return "ok";
+        case OPMX_ERR_BAD_ARGUMENT: return "bad argument";
+        case OPMX_ERR_UNSUPPORTED: return "unsupported dtype, expert count or experts-per-token";
+        case OPMX_ERR_WORKSPACE: return "workspace missing or too small";
+        case OPMX_ERR_ALIGNMENT: return "pointer or row pitch not aligned";
+        case OPMX_ERR_LAUNCH: return "HIP launch failed";
+    }
+    return "unknown status";
+}
+
+int opmx_linear(const void *X, const void *W, const void *B, int64_t T, int64_t K, int64_t N, int dtype,
+                void *Y, void *stream)
+{
+    if (T < 0 || K < 0 || N < 0) return OPMX_ERR_BAD_ARGUMENT;
+    if (!dtype_ok(dtype)) return OPMX_ERR_UNSUPPORTED;
+    if (T == 0 || N == 0) return OPMX_OK;
+    if (!X || !W || !Y || K == 0) return OPMX_ERR_BAD_ARGUMENT;
+    return launch_linear(X, W, B, T, K, N, dtype, Y, st(stream));
+}
+
+size_t opmx_moe_select_workspace_bytes(int64_t T, int E, int k) { return moe_select_workspace_bytes(T, E, k); }
+
+int opmx_moe_select(const void *X, const void *scores, int64_t T, int64_t H, int E, int k, int dtype,
+                    void *X_expand_permute, void *expert_weights, int64_t *invert_permutation,
+                    int64_t *expert_offset, int32_t *expert_ids, void *workspace, size_t workspace_bytes,
+                    void *stream)
+{
+    if (T < 0 || H < 0 || E <= 0 || k <= 0 || k > E) return OPMX_ERR_BAD_ARGUMENT;
+    if (!dtype_ok(dtype) || E > OPMX_MOE_MAX_EXPERTS || k > OPMX_MOE_MAX_EXPERTS_PER_TOKEN)
+        return OPMX_ERR_UNSUPPORTED;
+    if (T > (int64_t{1} << 31) / k) return OPMX_ERR_UNSUPPORTED;
+    if (!expert_offset) return OPMX_ERR_BAD_ARGUMENT;
+    if (T > 0 && (!scores || !expert_weights || !invert_permutation)) return OPMX_ERR_BAD_ARGUMENT;
+    if (T > 0 && H > 0 && (!X || !X_expand_permute)) return OPMX_ERR_BAD_ARGUMENT;
+    if (T > 0 && (!workspace || workspace_bytes < moe_select_workspace_bytes(T, E, k))) return OPMX_ERR_WORKSPACE;
+    if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 255u)) return OPMX_ERR_ALIGNMENT;
+    return launch_moe_select(X, scores, T, H, E, k, dtype, X_expand_permute, expert_weights, invert_permutation,
+                             expert_offset, expert_ids, workspace, st(stream));
+}
+
+size_t opmx_moe_grouped_gemm_workspace_bytes(int E, int64_t R, int64_t K, int64_t N, int dtype)
+{
+    return grouped_gemm_workspace_bytes(E, R, K, N, dtype);
+}
+
+static int grouped_checked(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
+                           int64_t K, int64_t N, int dtype, int epilogue, int64_t hint, void *Y, void *ws,
+                           size_t ws_bytes, void *stream)
+{
+    if (E <= 0 || R < 0 || K < 0 || N < 0) return OPMX_ERR_BAD_ARGUMENT;
+    if (!dtype_ok(dtype) || E > OPMX_MOE_MAX_EXPERTS) return OPMX_ERR_UNSUPPORTED;
+    if (epilogue != OPMX_EPILOGUE_NONE && epilogue != OPMX_EPILOGUE_SWIGLU) return OPMX_ERR_BAD_ARGUMENT;
+    if (epilogue == OPMX_EPILOGUE_SWIGLU && N % 2) return OPMX_ERR_BAD_ARGUMENT;
+    if (R == 0 || N == 0) return OPMX_OK;
+    if (!X || !off || !W || !Y || K == 0) return OPMX_ERR_BAD_ARGUMENT;
+    return launch_grouped_gemm(X, off, W, B, E, R, K, N, dtype, epilogue, hint, Y, ws, ws_bytes, st(stream));
+}
+
+int opmx_moe_column_parallel_linear(const void *X, const int64_t *expert_offset, const void *W, const void *B,
+                                    int E, int64_t R, int64_t K, int64_t N, int dtype, int epilogue,
+                                    int64_t rows_per_expert_hint, void *Y, void *workspace,
+                                    size_t workspace_bytes, void *stream)
+{
+    return grouped_checked(X, expert_offset, W, B, E, R, K, N, dtype, epilogue, rows_per_expert_hint, Y,
+                           workspace, workspace_bytes, stream);
+}
+
+int opmx_moe_row_parallel_linear(const void *X, const int64_t *expert_offset, const void *W, const void *B,
+                                 int E, int64_t R, int64_t K, int64_t N, int dtype,
+                                 int64_t rows_per_expert_hint, void *Y, void *workspace, size_t workspace_bytes,
+                                 void *stream)
+{
+    return grouped_checked(X, expert_offset, W, B, E, R, K, N, dtype, OPMX_EPILOGUE_NONE, rows_per_expert_hint,
+                           Y, workspace, workspace_bytes, stream);
+}
+
+int opmx_swiglu(const void *X, int64_t R, int64_t D, float beta, int dtype, void *Y, void *stream)
+{
+    if (R < 0 || D < 0) return OPMX_ERR_BAD_ARGUMENT;
+    if (!dtype_ok(dtype)) return OPMX_ERR_UNSUPPORTED;
+    if (R == 0 || D == 0) return OPMX_OK;
+    if (!X || !Y) return OPMX_ERR_BAD_ARGUMENT;
+    return launch_swiglu(X, R, D, beta, dtype, Y, st(stream));
+}
+
+int opmx_silu(const void *X, const void *gate, int64_t n, int dtype, void *Y, void *stream)
+{
+    if (n < 0) return OPMX_ERR_BAD_ARGUMENT;
+    if (!dtype_ok(dtype)) return OPMX_ERR_UNSUPPORTED;
+    if (n == 0) return OPMX_OK;
+    if (!X || !Y) return OPMX_ERR_BAD_ARGUMENT;
+    return launch_silu(X, gate, n, dtype, Y, st(stream));
+}
+
+int opmx_moe_reduce(const void *Y, const void *expert_weights, const int64_t *invert_permutation, int64_t T,
+                    int k, int64_t N, int dtype, void *out, void *stream)
+{
+    if (T < 0 || N < 0 || k <= 0) return OPMX_ERR_BAD_ARGUMENT;
+    if (!dtype_ok(dtype) || k > OPMX_MOE_MAX_EXPERTS_PER_TOKEN) return OPMX_ERR_UNSUPPORTED;
+    if (T == 0 || N == 0) return OPMX_OK;
+    if (!Y || !expert_weights || !invert_permutation || !out) return OPMX_ERR_BAD_ARGUMENT;
+    return launch_moe_reduce(Y, expert_weights, invert_permutation, T, k, N, dtype, out, st(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,76 @@
+// Shared device helpers for the OPMX MoE kernels (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "opmx_moe.h"
+
+namespace opmx {
+
+using f16 = _Float16;
+using bf16 = __bf16;
+
+constexpr int kWave = 64;
+
+template <typename T> struct DType;
+template <> struct DType<float> { static constexpr int id = OPMX_DTYPE_F32; };
+template <> struct DType<f16> { static constexpr int id = OPMX_DTYPE_F16; };
+template <> struct DType<bf16> { static constexpr int id = OPMX_DTYPE_BF16; };
+
+template <typename T> __device__ __forceinline__ float to_f32(T v) { return static_cast<float>(v); }
+template <typename T> __device__ __forceinline__ T from_f32(float v) { return static_cast<T>(v); }  // RNE
+
+// 16-byte vector of T.
+template <typename T> struct Vec16 {
+    static constexpr int n = 16 / sizeof(T);
+    T v[n];
+};
+template <typename T> __device__ __forceinline__ Vec16<T> load16(const T *p)
+{
+    Vec16<T> r;
+    *reinterpret_cast<uint4 *>(&r) = *reinterpret_cast<const uint4 *>(p);
+    return r;
+}
+template <typename T> __device__ __forceinline__ void store16(T *p, const Vec16<T> &r)
+{
+    *reinterpret_cast<uint4 *>(p) = *reinterpret_cast<const uint4 *>(&r);
+}
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
+
+// Butterfly sum over the 64 lanes of a wave; every lane gets the total.
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, kWave);
+    return v;
+}
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+#define OPMX_LAUNCH_CHECK()                                   \
+    do {                                                      \
+        if (hipGetLastError() != hipSuccess) return OPMX_ERR_LAUNCH; \
+    } while (0)
+
+// Host launchers (one per translation unit); all return an opmx_status.
+int launch_linear(const void *X, const void *W, const void *B, int64_t T, int64_t K, int64_t N,
+                  int dtype, void *Y, hipStream_t s);
+int launch_moe_select(const void *X, const void *scores, int64_t T, int64_t H, int E, int k, int dtype,
+                      void *Xp, void *w, int64_t *inv, int64_t *off, int32_t *ids, void *ws,
+                      hipStream_t s);
+size_t moe_select_workspace_bytes(int64_t T, int E, int k);
+int launch_swiglu(const void *X, int64_t R, int64_t D, float beta, int dtype, void *Y, hipStream_t s);
+int launch_silu(const void *X, const void *gate, int64_t n, int dtype, void *Y, hipStream_t s);
+int launch_moe_reduce(const void *Y, const void *w, const int64_t *inv, int64_t T, int k, int64_t N,
+                      int dtype, void *out, hipStream_t s);
+int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const void *B, int E,
+                        int64_t R, int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint,
+                        void *Y, void *ws, size_t ws_bytes, hipStream_t s);
+size_t grouped_gemm_workspace_bytes(int E, int64_t R, int64_t K, int64_t N, int dtype);
+
+}  // namespace opmx

@@ -1,0 +1,115 @@
+// Skinny linear for gfx950: Y = X W^T (+B) with few output features (the MoE
+// router gate, N = number of experts).  HBM bound on X: every block streams its
+// tokens' rows once with 16-byte loads and keeps W in cache.
+// Semantics: torch_function/Linear.py:32 of OpenPPL/ppl.pmx.
+#include "common.h"
+
+namespace opmx {
+namespace {
+
+constexpr int kNT = 8;   // output features per pass
+
+template <typename T, int TPB, bool VEC>
+__global__ __launch_bounds__(256) void linear_kernel(const T *__restrict__ X, const T *__restrict__ W,
+                                                     const T *__restrict__ B, int64_t Ttok, int64_t K, int64_t N,
+                                                     T *__restrict__ Y)
+{
+    constexpr int n = VEC ? Vec16<T>::n : 1;
+    __shared__ float red[256 / kWave][TPB * kNT];
+    const int64_t t0 = static_cast<int64_t>(blockIdx.x) * TPB;
+    const int lane = lane_id(), wave = threadIdx.x / kWave;
+
+    for (int64_t n0 = 0; n0 < N; n0 += kNT) {
+        float acc[TPB][kNT];
+#pragma unroll
+        for (int a = 0; a < TPB; ++a)
+#pragma unroll
+            for (int j = 0; j < kNT; ++j) acc[a][j] = 0.0f;
+
+        for (int64_t c = static_cast<int64_t>(threadIdx.x) * n; c < K; c += 256 * n) {
+            float xv[TPB][n];
+#pragma unroll
+            for (int a = 0; a < TPB; ++a) {
+                const int64_t t = t0 + a < Ttok ? t0 + a : Ttok - 1;
+                if (VEC) {
+                    Vec16<T> v = load16(X + t * K + c);
+#pragma unroll
+                    for (int i = 0; i < n; ++i) xv[a][i] = to_f32(v.v[i]);
+                } else {
+                    xv[a][0] = to_f32(X[t * K + c]);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < kNT; ++j) {
+                const int64_t row = n0 + j < N ? n0 + j : N - 1;
+                float wv[n];
+                if (VEC) {
+                    Vec16<T> v = load16(W + row * K + c);
+#pragma unroll
+                    for (int i = 0; i < n; ++i) wv[i] = to_f32(v.v[i]);
+                } else {
+                    wv[0] = to_f32(W[row * K + c]);
+                }
+#pragma unroll
+                for (int a = 0; a < TPB; ++a)
+#pragma unroll
+                    for (int i = 0; i < n; ++i) acc[a][j] += xv[a][i] * wv[i];
+            }
+        }
+#pragma unroll
+        for (int a = 0; a < TPB; ++a)
+#pragma unroll
+            for (int j = 0; j < kNT; ++j) {
+                float v = wave_sum(acc[a][j]);
+                if (lane == 0) red[wave][a * kNT + j] = v;
+            }
+        __syncthreads();
+        if (threadIdx.x < TPB * kNT) {
+            const int a = threadIdx.x / kNT, j = threadIdx.x % kNT;
+            if (t0 + a < Ttok && n0 + j < N) {
+                float v = 0.0f;
+#pragma unroll
+                for (int w = 0; w < 256 / kWave; ++w) v += red[w][threadIdx.x];
+                if (B) v += to_f32(B[n0 + j]);
+                Y[(t0 + a) * N + n0 + j] = from_f32<T>(v);
+            }
+        }
+        __syncthreads();
+    }
+}
+
+template <typename T>
+int linear_impl(const void *X_, const void *W_, const void *B_, int64_t Ttok, int64_t K, int64_t N, void *Y_,
+                hipStream_t s)
+{
+    if (Ttok == 0 || N == 0) return OPMX_OK;
+    const T *X = static_cast<const T *>(X_), *W = static_cast<const T *>(W_), *B = static_cast<const T *>(B_);
+    T *Y = static_cast<T *>(Y_);
+    const bool vec = K % Vec16<T>::n == 0 && aligned16(X) && aligned16(W);
+    if (Ttok >= 1024) {
+        const unsigned grid = static_cast<unsigned>(ceil_div(Ttok, 4));
+        if (vec) linear_kernel<T, 4, true><<<grid, 256, 0, s>>>(X, W, B, Ttok, K, N, Y);
+        else linear_kernel<T, 4, false><<<grid, 256, 0, s>>>(X, W, B, Ttok, K, N, Y);
+    } else {
+        const unsigned grid = static_cast<unsigned>(Ttok);
+        if (vec) linear_kernel<T, 1, true><<<grid, 256, 0, s>>>(X, W, B, Ttok, K, N, Y);
+        else linear_kernel<T, 1, false><<<grid, 256, 0, s>>>(X, W, B, Ttok, K, N, Y);
+    }
+    OPMX_LAUNCH_CHECK();
+    return OPMX_OK;
+}
+
+}  // namespace
+
+int launch_linear(const void *X, const void *W, const void *B, int64_t T, int64_t K, int64_t N, int dtype,
+                  void *Y, hipStream_t s)
+{
+    switch (dtype) {
+        case OPMX_DTYPE_F32: return linear_impl<float>(X, W, B, T, K, N, Y, s);
+        case OPMX_DTYPE_F16: return linear_impl<f16>(X, W, B, T, K, N, Y, s);
+        case OPMX_DTYPE_BF16: return linear_impl<bf16>(X, W, B, T, K, N, Y, s);
+    }
+    return OPMX_ERR_UNSUPPORTED;
+}
+
+}  // namespace opmx

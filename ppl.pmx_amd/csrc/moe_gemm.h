@@ -1,0 +1,109 @@
+// Pieces shared by the grouped-GEMM kernels: the on-device tile scheduler that
+// turns expert_offset into (expert, row range) work items without a host sync,
+// MFMA fragment types and the zero-fill of rows no expert owns.
+#pragma once
+#include "common.h"
+
+namespace opmx {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+template <typename T> struct Mfma;
+template <> struct Mfma<f16> {
+    using frag = half8_t;
+    static __device__ __forceinline__ float16_t m32(frag a, frag b, float16_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float4_t m16(frag a, frag b, float4_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct Mfma<bf16> {
+    using frag = bf16x8_t;
+    static __device__ __forceinline__ float16_t m32(frag a, frag b, float16_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float4_t m16(frag a, frag b, float4_t c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+};
+
+// One unit of grouped-GEMM work: `rows` rows starting at `row0`, all of expert `e`.
+struct MTile {
+    int e;
+    int rows;        // 0 => no work for this block
+    int64_t row0;
+};
+
+// Copies expert_offset into LDS (clamped to a non-decreasing sequence inside
+// [0, R], so a corrupt offset can never send a store outside Y) and finds the
+// `tile`-th row tile of height BM in expert order.  s_off needs E+1 entries.
+// Every thread of the block must call it; it contains block barriers.
+__device__ __forceinline__ MTile find_mtile(const int64_t *__restrict__ off, int E, int64_t R, int BM,
+                                            int64_t tile, int64_t *s_off)
+{
+    for (int i = threadIdx.x; i <= E; i += blockDim.x) {
+        int64_t v = off[i];
+        s_off[i] = v < 0 ? 0 : (v > R ? R : v);
+    }
+    __syncthreads();
+    MTile t;
+    t.e = 0;
+    t.rows = 0;
+    t.row0 = 0;
+    int64_t prev = s_off[0];
+    for (int e = 0; e < E; ++e) {
+        int64_t lo = prev, hi = s_off[e + 1];
+        if (hi < lo) hi = lo;
+        const int64_t nt = (hi - lo + BM - 1) / BM;
+        if (tile < nt) {
+            t.e = e;
+            t.row0 = lo + tile * BM;
+            const int64_t left = hi - t.row0;
+            t.rows = static_cast<int>(left < BM ? left : BM);
+            return t;
+        }
+        tile -= nt;
+        prev = hi;
+    }
+    return t;
+}
+
+// Upper bound of the number of row tiles for any offsets: sum ceil(m_e/BM) <= R/BM + E.
+inline int64_t max_mtiles(int64_t R, int E, int BM) { return R / BM + E; }
+
+// Rows outside [off[0], off[E]) belong to no expert and must read as zero
+// (MoeColumnParallelLinear.py:59 starts from torch.zeros).  Normally there are
+// none and this is two loads.  Work is shared by all blocks of the grid.
+template <typename T>
+__device__ __forceinline__ void zero_unowned_rows(T *__restrict__ Y, int64_t R, int64_t ncols,
+                                                  const int64_t *__restrict__ off, int E)
+{
+    int64_t lo = off[0], hi = off[E];
+    lo = lo < 0 ? 0 : (lo > R ? R : lo);
+    hi = hi < lo ? lo : (hi > R ? R : hi);
+    const int64_t head = lo * ncols, tail0 = hi * ncols, total = R * ncols;
+    if (head == 0 && tail0 == total) return;
+    const int64_t nb = static_cast<int64_t>(gridDim.x) * gridDim.y * gridDim.z;
+    const int64_t b = blockIdx.x + static_cast<int64_t>(gridDim.x) * (blockIdx.y + static_cast<int64_t>(gridDim.y) * blockIdx.z);
+    const int64_t stride = nb * blockDim.x;
+    for (int64_t i = b * blockDim.x + threadIdx.x; i < head; i += stride) Y[i] = from_f32<T>(0.0f);
+    for (int64_t i = tail0 + b * blockDim.x + threadIdx.x; i < total; i += stride) Y[i] = from_f32<T>(0.0f);
+}
+
+int launch_gemm_generic(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
+                        int64_t K, int64_t N, int dtype, int epilogue, void *Y, hipStream_t s);
+int launch_gemm_tiled(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
+                      int64_t K, int64_t N, int dtype, int epilogue, int variant, void *Y, hipStream_t s);
+int launch_gemm_stream(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
+                       int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint, int variant, void *Y,
+                       hipStream_t s);
+
+}  // namespace opmx

@@ -1,0 +1,189 @@
+// Grouped expert GEMM for gfx950, HBM-bound regime (few rows per expert: decode).
+//
+// The job is to read every active expert's W[e] [N,K] exactly once at HBM speed;
+// the flops ride along on v_mfma_f32_16x16x32 with W as the A operand (16 weight
+// rows per wave) and the expert's few X rows as the B operand.
+//
+//  * a block = 4 waves = 64 consecutive rows of W[e] (one 16-row group per wave)
+//    x one row tile (<= 16*MT rows) of expert e, over the whole K;
+//  * W is fetched with fully coalesced 16-byte loads (a wave instruction reads
+//    1 KiB contiguous), one K-chunk ahead in registers, then transposed into the
+//    MFMA operand layout through a wave-private LDS strip (no block barrier);
+//  * the X chunk is shared by the four waves through double-buffered LDS: one
+//    barrier per K-chunk;
+//  * experts with no rows produce no work, so their weights are never touched.
+// Semantics: torch_function/MoeColumnParallelLinear.py:61-67 and
+// torch_function/MoeRowParallelLinear.py:47-53 of OpenPPL/ppl.pmx.
+#include "moe_gemm.h"
+
+namespace opmx {
+namespace {
+
+constexpr int SW = 4;            // waves per block
+constexpr int SROWS = 16 * SW;   // W rows per block
+
+template <typename T, int MT, int KC>
+__global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restrict__ X,
+                                                               const int64_t *__restrict__ off,
+                                                               const T *__restrict__ W,
+                                                               const T *__restrict__ Bias, int E, int64_t R,
+                                                               int64_t K, int64_t N, T *__restrict__ Y)
+{
+    constexpr int RS = KC * 2 + 16;              // LDS row stride in bytes (pad 16: conflict-free strips)
+    constexpr int RPL = 512 / KC;                // W rows covered by one wave load (1 KiB)
+    constexpr int NLW = 16 / RPL;                // W loads per wave per chunk
+    constexpr int XM = 16 * MT;                  // X rows per tile
+    constexpr int CPR = KC / 8;                  // 16-byte chunks per row per K-chunk
+    constexpr int NLX = XM * CPR / (SW * 64);    // X loads per thread per chunk
+    constexpr int WSTRIP = 16 * RS;
+    constexpr int XBUF = XM * RS;
+    static_assert(XM * CPR % (SW * 64) == 0, "X chunk must divide over the block");
+    using frag = typename Mfma<T>::frag;
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];   // [SW][WSTRIP] | [2][XBUF]
+    __shared__ int64_t s_off[OPMX_MOE_MAX_EXPERTS + 1];
+
+    zero_unowned_rows(Y, R, N, off, E);
+    const MTile mt = find_mtile(off, E, R, XM, blockIdx.y, s_off);
+    if (mt.rows == 0) return;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    char *wstrip = smem + wave * WSTRIP;
+    char *xbuf = smem + SW * WSTRIP;
+
+    // ---- this wave's 16 rows of W[e]; rows past N are clamped (masked at the store)
+    const int64_t nbase = static_cast<int64_t>(blockIdx.x) * SROWS + wave * 16;
+    const T *We = W + static_cast<int64_t>(mt.e) * N * K;
+    const int wl_row = lane / (64 / RPL);               // row inside one wave load
+    const int wl_k = (lane % (64 / RPL)) * 8;           // k offset inside the chunk
+    const T *wsrc[NLW];
+    int wdst[NLW];
+#pragma unroll
+    for (int i = 0; i < NLW; ++i) {
+        const int row = i * RPL + wl_row;
+        int64_t n = nbase + row;
+        n = n < N ? n : N - 1;
+        wsrc[i] = We + n * K + wl_k;
+        wdst[i] = row * RS + wl_k * 2;
+    }
+    // ---- this thread's share of the X chunk
+    const T *xsrc[NLX];
+    int xdst[NLX], xk[NLX];
+#pragma unroll
+    for (int i = 0; i < NLX; ++i) {
+        const int q = tid + SW * 64 * i, row = q / CPR, c = q % CPR;
+        const int r = row < mt.rows ? row : mt.rows - 1;
+        xsrc[i] = X + (mt.row0 + r) * K + c * 8;
+        xdst[i] = row * RS + c * 16;
+        xk[i] = c * 8;
+    }
+
+    float4_t acc[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[m] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+    uint4 wreg[NLW], xreg[NLX];
+    auto fetch = [&](int64_t k0) {
+#pragma unroll
+        for (int i = 0; i < NLW; ++i)
+            wreg[i] = (k0 + wl_k < K) ? *reinterpret_cast<const uint4 *>(wsrc[i] + k0) : zero4;
+#pragma unroll
+        for (int i = 0; i < NLX; ++i)
+            xreg[i] = (k0 + xk[i] < K) ? *reinterpret_cast<const uint4 *>(xsrc[i] + k0) : zero4;
+    };
+
+    const int nchunks = static_cast<int>((K + KC - 1) / KC);
+    fetch(0);
+    const int fr = lane & 15, fg = lane >> 4;   // fragment row (W row / X row) and k group
+    for (int kc = 0; kc < nchunks; ++kc) {
+        char *xcur = xbuf + (kc & 1) * XBUF;
+#pragma unroll
+        for (int i = 0; i < NLW; ++i) *reinterpret_cast<uint4 *>(wstrip + wdst[i]) = wreg[i];
+#pragma unroll
+        for (int i = 0; i < NLX; ++i) *reinterpret_cast<uint4 *>(xcur + xdst[i]) = xreg[i];
+        if (kc + 1 < nchunks) fetch(static_cast<int64_t>(kc + 1) * KC);
+        __syncthreads();
+#pragma unroll
+        for (int s = 0; s < KC / 32; ++s) {
+            const int c = s * 4 + fg;
+            const frag a = *reinterpret_cast<const frag *>(wstrip + fr * RS + c * 16);
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                if (m * 16 < mt.rows) {
+                    const frag b = *reinterpret_cast<const frag *>(xcur + (m * 16 + fr) * RS + c * 16);
+                    acc[m] = Mfma<T>::m16(a, b, acc[m]);
+                }
+            }
+        }
+    }
+
+    // acc[m][i]: W row nbase + fg*4 + i, X row m*16 + fr
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int row = m * 16 + fr;
+        if (row >= mt.rows) continue;
+        T *yrow = Y + (mt.row0 + row) * N;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int64_t n = nbase + fg * 4 + i;
+            if (n >= N) continue;
+            float v = acc[m][i];
+            if (Bias) v += to_f32(Bias[static_cast<int64_t>(mt.e) * N + n]);
+            yrow[n] = from_f32<T>(v);
+        }
+    }
+}
+
+template <typename T, int MT, int KC>
+int stream_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
+                  int64_t N, void *Y, hipStream_t s)
+{
+    constexpr int RS = KC * 2 + 16;
+    constexpr int smem = SW * 16 * RS + 2 * 16 * MT * RS;
+    auto kern = gemm_stream_kernel<T, MT, KC>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                smem) != hipSuccess)
+            return OPMX_ERR_LAUNCH;
+        attr_done = true;
+    }
+    dim3 grid(static_cast<unsigned>(ceil_div(N, SROWS)), static_cast<unsigned>(max_mtiles(R, E, 16 * MT)));
+    kern<<<grid, SW * 64, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
+                                     static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y));
+    OPMX_LAUNCH_CHECK();
+    return OPMX_OK;
+}
+
+template <typename T>
+int stream_impl(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
+                int64_t N, int64_t rows_hint, int variant, void *Y, hipStream_t s)
+{
+    const int64_t m = rows_hint > 0 ? rows_hint : R;
+    if (variant == 1) {   // 512-wide K chunks
+        if (m <= 16) return stream_launch<T, 1, 512>(X, off, W, B, E, R, K, N, Y, s);
+        if (m <= 32) return stream_launch<T, 2, 512>(X, off, W, B, E, R, K, N, Y, s);
+        return stream_launch<T, 4, 256>(X, off, W, B, E, R, K, N, Y, s);
+    }
+    if (m <= 16) return stream_launch<T, 1, 256>(X, off, W, B, E, R, K, N, Y, s);
+    if (m <= 32) return stream_launch<T, 2, 256>(X, off, W, B, E, R, K, N, Y, s);
+    return stream_launch<T, 4, 256>(X, off, W, B, E, R, K, N, Y, s);
+}
+
+}  // namespace
+
+// Requires: dtype f16/bf16, K % 8 == 0, 16-byte aligned X and W.  Epilogue NONE only.
+int launch_gemm_stream(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
+                       int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint, int variant, void *Y,
+                       hipStream_t s)
+{
+    if (epilogue != OPMX_EPILOGUE_NONE) return OPMX_ERR_UNSUPPORTED;
+    switch (dtype) {
+        case OPMX_DTYPE_F16: return stream_impl<f16>(X, off, W, B, E, R, K, N, rows_hint, variant, Y, s);
+        case OPMX_DTYPE_BF16: return stream_impl<bf16>(X, off, W, B, E, R, K, N, rows_hint, variant, Y, s);
+    }
+    return OPMX_ERR_UNSUPPORTED;
+}
+
+}  // namespace opmx

@@ -1,0 +1,221 @@
+// Grouped expert GEMM for gfx950, MFMA-bound regime (many rows per expert).
+//
+//   Y[r, :] = X[r, :] W[e]^T (+ B[e])   for off[e] <= r < off[e+1]
+//
+// X [R,K] and W[e] [N,K] are both K-contiguous, so A and B fragments of
+// v_mfma_f32_32x32x16_{f16,bf16} are 16-byte loads.  A block owns a BM x BN
+// output tile of ONE expert (tiles never straddle experts; the tile list is
+// derived on the device from expert_offset, no host sync), stages X and W
+// tiles of BK=64 through XOR-swizzled LDS with register prefetch (two LDS
+// buffers, one barrier per k-tile) and accumulates in fp32.  Optional SwiGLU
+// epilogue on the accumulators (gate rows i and up rows N/2+i of W are placed
+// in the same lane by the B-tile row order).
+// Semantics: torch_function/MoeColumnParallelLinear.py:61-67,
+// torch_function/MoeRowParallelLinear.py:47-53, torch_function/SwiGLU.py:15-16.
+#include "moe_gemm.h"
+
+namespace opmx {
+namespace {
+
+constexpr int BK = 64;                 // k elements per LDS tile (128 bytes per row)
+constexpr int ROWB = BK * 2;           // bytes per LDS row
+constexpr int CH = ROWB / 16;          // 16-byte chunks per row (8)
+
+__device__ __forceinline__ int lds_off(int row, int chunk) { return row * ROWB + ((chunk ^ (row & 7)) << 4); }
+
+template <typename T, int BM, int BN, int WM, int WN, bool SWIGLU>
+__global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__restrict__ X,
+                                                                  const int64_t *__restrict__ off,
+                                                                  const T *__restrict__ W,
+                                                                  const T *__restrict__ Bias, int E, int64_t R,
+                                                                  int64_t K, int64_t N, T *__restrict__ Y)
+{
+    constexpr int NT = WM * WN * 64;
+    constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
+    constexpr int BNO = SWIGLU ? BN / 2 : BN;            // output columns per tile
+    constexpr int LA = BM * CH / NT, LB = BN * CH / NT;  // 16-byte loads per thread per k-tile
+    constexpr int STAGE = (BM + BN) * ROWB;
+    static_assert(BM * CH % NT == 0 && BN * CH % NT == 0, "tile/threads mismatch");
+    static_assert(!SWIGLU || TN % 2 == 0, "SwiGLU needs an even number of n sub-tiles per wave");
+    using frag = typename Mfma<T>::frag;
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    __shared__ int64_t s_off[OPMX_MOE_MAX_EXPERTS + 1];
+
+    const int64_t ncols = SWIGLU ? N / 2 : N;
+    zero_unowned_rows(Y, R, ncols, off, E);
+    const MTile mt = find_mtile(off, E, R, BM, blockIdx.y, s_off);
+    if (mt.rows == 0) return;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int64_t n0 = static_cast<int64_t>(blockIdx.x) * BNO;
+    const T *Xt = X + mt.row0 * K;
+    const T *We = W + static_cast<int64_t>(mt.e) * N * K;
+
+    // per-thread global offsets (elements) and LDS offsets (bytes) of its loads
+    int a_src[LA], a_dst[LA], b_src[LB], b_dst[LB];
+#pragma unroll
+    for (int i = 0; i < LA; ++i) {
+        const int q = tid + NT * i, row = q / CH, c = q % CH;
+        const int r = row < mt.rows ? row : mt.rows - 1;
+        a_src[i] = static_cast<int>(r * K + c * 8);
+        a_dst[i] = lds_off(row, c);
+    }
+#pragma unroll
+    for (int i = 0; i < LB; ++i) {
+        const int q = tid + NT * i, row = q / CH, c = q % CH;
+        int64_t wrow;
+        if (SWIGLU) {
+            const int w = row / WTN, jj = row % WTN, half = jj / (WTN / 2);
+            int64_t ii = n0 + w * (WTN / 2) + jj % (WTN / 2);
+            ii = ii < ncols ? ii : ncols - 1;
+            wrow = half * ncols + ii;
+        } else {
+            wrow = n0 + row < N ? n0 + row : N - 1;
+        }
+        b_src[i] = static_cast<int>(wrow * K + c * 8);
+        b_dst[i] = BM * ROWB + lds_off(row, c);
+    }
+
+    float16_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    uint4 ra[LA], rb[LB];
+    const int nk = static_cast<int>(K / BK);
+#pragma unroll
+    for (int i = 0; i < LA; ++i) ra[i] = *reinterpret_cast<const uint4 *>(Xt + a_src[i]);
+#pragma unroll
+    for (int i = 0; i < LB; ++i) rb[i] = *reinterpret_cast<const uint4 *>(We + b_src[i]);
+#pragma unroll
+    for (int i = 0; i < LA; ++i) *reinterpret_cast<uint4 *>(smem + a_dst[i]) = ra[i];
+#pragma unroll
+    for (int i = 0; i < LB; ++i) *reinterpret_cast<uint4 *>(smem + b_dst[i]) = rb[i];
+    __syncthreads();
+
+    const int lrow = lane & 31, lk = lane >> 5;
+    for (int kt = 0; kt < nk; ++kt) {
+        const char *cur = smem + (kt & 1) * STAGE;
+        char *nxt = smem + ((kt + 1) & 1) * STAGE;
+        const bool more = kt + 1 < nk;
+        if (more) {
+            const int64_t ko = static_cast<int64_t>(kt + 1) * BK;
+#pragma unroll
+            for (int i = 0; i < LA; ++i) ra[i] = *reinterpret_cast<const uint4 *>(Xt + a_src[i] + ko);
+#pragma unroll
+            for (int i = 0; i < LB; ++i) rb[i] = *reinterpret_cast<const uint4 *>(We + b_src[i] + ko);
+        }
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            frag fa[TM], fb[TN];
+            const int chunk = ks * 2 + lk;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                fa[i] = *reinterpret_cast<const frag *>(cur + lds_off(wm * WTM + i * 32 + lrow, chunk));
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                fb[j] = *reinterpret_cast<const frag *>(cur + BM * ROWB + lds_off(wn * WTN + j * 32 + lrow, chunk));
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::m32(fa[i], fb[j], acc[i][j]);
+        }
+        if (more) {
+#pragma unroll
+            for (int i = 0; i < LA; ++i) *reinterpret_cast<uint4 *>(nxt + a_dst[i]) = ra[i];
+#pragma unroll
+            for (int i = 0; i < LB; ++i) *reinterpret_cast<uint4 *>(nxt + b_dst[i]) = rb[i];
+        }
+        __syncthreads();
+    }
+
+    // epilogue: acc[i][j][v] is row (v/4)*8 + (lane/32)*4 + v%4, column lane%32 of its 32x32 sub-tile
+    const T *be = Bias ? Bias + static_cast<int64_t>(mt.e) * N : nullptr;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < (SWIGLU ? TN / 2 : TN); ++j) {
+            const int64_t n = SWIGLU ? n0 + wn * (WTN / 2) + j * 32 + lrow : n0 + wn * WTN + j * 32 + lrow;
+            if (n >= ncols) continue;
+            const float bg = be ? to_f32(be[n]) : 0.0f;
+            const float bu = (SWIGLU && be) ? to_f32(be[ncols + n]) : 0.0f;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = wm * WTM + i * 32 + (v / 4) * 8 + lk * 4 + (v % 4);
+                if (row >= mt.rows) continue;
+                float val = acc[i][j][v] + bg;
+                if (SWIGLU) {
+                    const float up = acc[i][j + TN / 2][v] + bu;
+                    val = up * val * sigmoidf_(val);
+                }
+                Y[(mt.row0 + row) * ncols + n] = from_f32<T>(val);
+            }
+        }
+}
+
+template <typename T, int BM, int BN, int WM, int WN>
+int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
+                 int64_t N, int epilogue, void *Y, hipStream_t s)
+{
+    constexpr int smem = 2 * (BM + BN) * ROWB;
+    const bool sw = epilogue == OPMX_EPILOGUE_SWIGLU;
+    const int64_t ncols = sw ? N / 2 : N;
+    dim3 grid(static_cast<unsigned>(ceil_div(ncols, sw ? BN / 2 : BN)), static_cast<unsigned>(max_mtiles(R, E, BM)));
+    dim3 block(WM * WN * 64);
+    static bool attr_done[2] = {false, false};
+    if (sw) {
+        auto kern = gemm_tiled_kernel<T, BM, BN, WM, WN, true>;
+        if (!attr_done[1]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    smem) != hipSuccess)
+                return OPMX_ERR_LAUNCH;
+            attr_done[1] = true;
+        }
+        kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y));
+    } else {
+        auto kern = gemm_tiled_kernel<T, BM, BN, WM, WN, false>;
+        if (!attr_done[0]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    smem) != hipSuccess)
+                return OPMX_ERR_LAUNCH;
+            attr_done[0] = true;
+        }
+        kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y));
+    }
+    OPMX_LAUNCH_CHECK();
+    return OPMX_OK;
+}
+
+template <typename T>
+int tiled_impl(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
+               int64_t N, int epilogue, int variant, void *Y, hipStream_t s)
+{
+    switch (variant) {
+        case 1: return tiled_launch<T, 256, 256, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        case 2: return tiled_launch<T, 256, 128, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        case 3: return tiled_launch<T, 256, 256, 2, 4>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        default: return tiled_launch<T, 128, 128, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+    }
+}
+
+}  // namespace
+
+// Requires: dtype f16/bf16, K % 64 == 0, 16-byte aligned X and W, N*K < 2^31.
+int launch_gemm_tiled(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
+                      int64_t K, int64_t N, int dtype, int epilogue, int variant, void *Y, hipStream_t s)
+{
+    switch (dtype) {
+        case OPMX_DTYPE_F16: return tiled_impl<f16>(X, off, W, B, E, R, K, N, epilogue, variant, Y, s);
+        case OPMX_DTYPE_BF16: return tiled_impl<bf16>(X, off, W, B, E, R, K, N, epilogue, variant, Y, s);
+    }
+    return OPMX_ERR_UNSUPPORTED;
+}
+
+}  // namespace opmx

@@ -1,0 +1,354 @@
+// MoeSelect for gfx950: top-k with ties to the lower expert id, softmax over the
+// picks, deterministic stable permutation by expert id, row expand/permute.
+// Semantics: torch_function/MoeSelect.py:37-64 of OpenPPL/ppl.pmx.
+//
+// Determinism: positions never come from an atomic counter.  A token's row is
+//   expert_offset[e] + (#tokens before it that picked e)
+// and the count is taken from bit matrices (one bit per (expert, token)), whose
+// construction by atomicOr is order independent.
+#include "common.h"
+
+namespace opmx {
+namespace {
+
+constexpr int kChunk = 256;          // tokens per routing block
+constexpr int kWords = kChunk / 32;  // bit-matrix words per expert
+constexpr int kMaxVpl = OPMX_MOE_MAX_EXPERTS / kWave;
+
+// Monotone map float -> uint32 (larger float => larger key).  NaN is the
+// largest key (torch.topk / torch.sort rank NaN first); -0.0 == +0.0.
+__device__ __forceinline__ uint32_t order_key(float f)
+{
+    if (f != f) return 0xFFFFFFFFu;
+    if (f == 0.0f) f = 0.0f;
+    uint32_t u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_value(uint32_t key)
+{
+    if (key == 0xFFFFFFFFu) return __uint_as_float(0x7FC00000u);
+    uint32_t u = (key & 0x80000000u) ? (key & 0x7FFFFFFFu) : ~key;
+    return __uint_as_float(u);
+}
+
+__device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int mask)
+{
+    uint32_t lo = __shfl_xor(static_cast<uint32_t>(v), mask, kWave);
+    uint32_t hi = __shfl_xor(static_cast<uint32_t>(v >> 32), mask, kWave);
+    return (static_cast<uint64_t>(hi) << 32) | lo;
+}
+
+// One group of G lanes (G a power of two, 8..64) routes one token.  Lane j < k
+// of the group ends up with the j-th pick and its softmax weight.
+template <typename T>
+__device__ __forceinline__ void route_token(const T *srow, int E, int k, int G, int vpl, int lig,
+                                            int &my_id, float &my_w)
+{
+    uint64_t keys[kMaxVpl];
+#pragma unroll
+    for (int v = 0; v < kMaxVpl; ++v) {
+        int e = lig + v * G;
+        keys[v] = (v < vpl && e < E)
+                      ? (static_cast<uint64_t>(order_key(to_f32(srow[e]))) << 32) | (0xFFFFFFFFu - e)
+                      : 0ull;
+    }
+    my_id = -1;
+    float my_v = 0.0f;
+    for (int j = 0; j < k; ++j) {
+        uint64_t best = keys[0];
+#pragma unroll
+        for (int v = 1; v < kMaxVpl; ++v) best = keys[v] > best ? keys[v] : best;
+        for (int m = G >> 1; m >= 1; m >>= 1) {
+            uint64_t o = shfl_xor_u64(best, m);
+            best = o > best ? o : best;
+        }
+        int wid = static_cast<int>(0xFFFFFFFFu - static_cast<uint32_t>(best));
+#pragma unroll
+        for (int v = 0; v < kMaxVpl; ++v)
+            if (lig + v * G == wid) keys[v] = 0ull;
+        if (lig == j) {
+            my_id = wid;
+            my_v = key_value(static_cast<uint32_t>(best >> 32));
+        }
+    }
+    // softmax over the k picked values (MoeSelect.py:41); pick 0 is the maximum
+    float vmax = __shfl(my_v, (lane_id() / G) * G, kWave);
+    float ev = (lig < k) ? expf(my_v - vmax) : 0.0f;
+    float sum = ev;
+    for (int m = G >> 1; m >= 1; m >>= 1) sum += __shfl_xor(sum, m, kWave);
+    my_w = ev / sum;
+}
+
+__device__ __forceinline__ void zero_bits(uint32_t *bits, int E)
+{
+    for (int i = threadIdx.x; i < E * kWords; i += blockDim.x) bits[i] = 0u;
+}
+
+// rank of token `tl` (chunk-local) among the chunk's tokens that picked e
+__device__ __forceinline__ int rank_in_chunk(const uint32_t *bits, const int *wordpre, int e, int tl)
+{
+    int w = tl >> 5;
+    return wordpre[e * kWords + w] + __popc(bits[e * kWords + w] & ((1u << (tl & 31)) - 1u));
+}
+
+// per expert: exclusive prefix of the word popcounts; returns nothing, fills
+// wordpre[e][w] and count[e]
+__device__ __forceinline__ void word_prefix(const uint32_t *bits, int *wordpre, int *count, int E)
+{
+    for (int e = threadIdx.x; e < E; e += blockDim.x) {
+        int run = 0;
+#pragma unroll
+        for (int w = 0; w < kWords; ++w) {
+            wordpre[e * kWords + w] = run;
+            run += __popc(bits[e * kWords + w]);
+        }
+        count[e] = run;
+    }
+}
+
+// ---- general path, kernel 1: top-k + weights + per-chunk expert histogram ----
+template <typename T>
+__global__ __launch_bounds__(kChunk) void select_topk_kernel(const T *__restrict__ scores, int64_t Ttok,
+                                                             int E, int k, int G, int vpl,
+                                                             T *__restrict__ weights,
+                                                             int32_t *__restrict__ ids,
+                                                             int32_t *__restrict__ hist)
+{
+    __shared__ uint32_t bits[OPMX_MOE_MAX_EXPERTS * kWords];
+    const int64_t t0 = static_cast<int64_t>(blockIdx.x) * kChunk;
+    const int lig = threadIdx.x % G, grp = threadIdx.x / G, ngrp = kChunk / G;
+    zero_bits(bits, E);
+    __syncthreads();
+    for (int tl = grp; tl < kChunk; tl += ngrp) {       // uniform trip count inside a wave
+        int64_t t = t0 + tl;
+        if (t < Ttok) {
+            int id;
+            float w;
+            route_token(scores + t * E, E, k, G, vpl, lig, id, w);
+            if (lig < k) {
+                ids[t * k + lig] = id;
+                weights[t * k + lig] = from_f32<T>(w);
+                atomicOr(&bits[id * kWords + (tl >> 5)], 1u << (tl & 31));
+            }
+        }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += blockDim.x) {
+        int c = 0;
+#pragma unroll
+        for (int w = 0; w < kWords; ++w) c += __popc(bits[e * kWords + w]);
+        hist[static_cast<int64_t>(blockIdx.x) * E + e] = c;
+    }
+}
+
+// ---- kernel 2: per expert exclusive scan over chunks, then offsets over experts ----
+__global__ __launch_bounds__(256) void select_scan_kernel(int32_t *__restrict__ hist, int nchunks, int E,
+                                                          int64_t R, int64_t *__restrict__ off)
+{
+    __shared__ int total[OPMX_MOE_MAX_EXPERTS];
+    const int lane = lane_id(), wave = threadIdx.x / kWave;
+    for (int e = wave; e < E; e += 256 / kWave) {
+        int running = 0;
+        for (int c0 = 0; c0 < nchunks; c0 += kWave) {
+            int c = c0 + lane;
+            int v = c < nchunks ? hist[static_cast<int64_t>(c) * E + e] : 0;
+            int incl = v;
+#pragma unroll
+            for (int d = 1; d < kWave; d <<= 1) {
+                int o = __shfl_up(incl, d, kWave);
+                if (lane >= d) incl += o;
+            }
+            if (c < nchunks) hist[static_cast<int64_t>(c) * E + e] = running + incl - v;
+            running += __shfl(incl, kWave - 1, kWave);
+        }
+        if (lane == 0) total[e] = running;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int64_t run = 0;
+        for (int e = 0; e < E; ++e) {
+            off[e] = run;                 // MoeSelect.py:54-59
+            run += total[e];
+        }
+        off[E] = R;                       // MoeSelect.py:60
+    }
+}
+
+// ---- kernel 3: rank inside the chunk -> invert_permutation ----
+__global__ __launch_bounds__(kChunk) void select_rank_kernel(const int32_t *__restrict__ ids,
+                                                             const int32_t *__restrict__ base,
+                                                             const int64_t *__restrict__ off, int64_t Ttok,
+                                                             int E, int k, int64_t *__restrict__ inv)
+{
+    __shared__ uint32_t bits[OPMX_MOE_MAX_EXPERTS * kWords];
+    __shared__ int wordpre[OPMX_MOE_MAX_EXPERTS * kWords];
+    __shared__ int count[OPMX_MOE_MAX_EXPERTS];
+    const int tl = threadIdx.x;
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * kChunk + tl;
+    zero_bits(bits, E);
+    __syncthreads();
+    if (t < Ttok)
+        for (int s = 0; s < k; ++s) atomicOr(&bits[ids[t * k + s] * kWords + (tl >> 5)], 1u << (tl & 31));
+    __syncthreads();
+    word_prefix(bits, wordpre, count, E);
+    __syncthreads();
+    if (t < Ttok)
+        for (int s = 0; s < k; ++s) {
+            int e = ids[t * k + s];
+            inv[t * k + s] = off[e] + base[static_cast<int64_t>(blockIdx.x) * E + e] +
+                             rank_in_chunk(bits, wordpre, e, tl);
+        }
+}
+
+// copy row X[t] to the k rows inv[t*k+s] of Xp
+template <typename T>
+__device__ __forceinline__ void expand_row(const T *__restrict__ X, T *__restrict__ Xp, int64_t t, int64_t H,
+                                           int k, const int64_t *inv_row, bool vec)
+{
+    const T *src = X + t * H;
+    if (vec) {
+        constexpr int n = Vec16<T>::n;
+        for (int64_t c = static_cast<int64_t>(threadIdx.x) * n; c < H; c += static_cast<int64_t>(blockDim.x) * n) {
+            Vec16<T> v = load16(src + c);
+            for (int s = 0; s < k; ++s) store16(Xp + inv_row[s] * H + c, v);
+        }
+    } else {
+        for (int64_t c = threadIdx.x; c < H; c += blockDim.x) {
+            T v = src[c];
+            for (int s = 0; s < k; ++s) Xp[inv_row[s] * H + c] = v;
+        }
+    }
+}
+
+// ---- kernel 4: X_expand_permute[inv[t,s]] = X[t]  (MoeSelect.py:45-47) ----
+template <typename T>
+__global__ __launch_bounds__(256) void select_expand_kernel(const T *__restrict__ X, T *__restrict__ Xp,
+                                                            const int64_t *__restrict__ inv, int64_t Ttok,
+                                                            int64_t H, int k, bool vec)
+{
+    for (int64_t t = blockIdx.x; t < Ttok; t += gridDim.x) expand_row(X, Xp, t, H, k, inv + t * k, vec);
+}
+
+// ---- small-T path: one launch.  Every block routes all T <= kChunk tokens
+// redundantly in LDS, then block b emits the outputs of token b and copies its row.
+template <typename T>
+__global__ __launch_bounds__(kChunk) void select_small_kernel(const T *__restrict__ X,
+                                                              const T *__restrict__ scores, int Ttok,
+                                                              int64_t H, int E, int k, int G, int vpl,
+                                                              T *__restrict__ Xp, T *__restrict__ weights,
+                                                              int64_t *__restrict__ inv,
+                                                              int64_t *__restrict__ off,
+                                                              int32_t *__restrict__ ids_out, bool vec)
+{
+    __shared__ uint32_t bits[OPMX_MOE_MAX_EXPERTS * kWords];
+    __shared__ int wordpre[OPMX_MOE_MAX_EXPERTS * kWords];
+    __shared__ int count[OPMX_MOE_MAX_EXPERTS + 1];
+    __shared__ int my_ids[OPMX_MOE_MAX_EXPERTS_PER_TOKEN];
+    __shared__ int64_t my_inv[OPMX_MOE_MAX_EXPERTS_PER_TOKEN];
+    const int lig = threadIdx.x % G, grp = threadIdx.x / G, ngrp = kChunk / G;
+    const int me = blockIdx.x;                 // the token this block emits
+    zero_bits(bits, E);
+    __syncthreads();
+    for (int tl = grp; tl < kChunk; tl += ngrp) {
+        if (tl < Ttok) {
+            int id;
+            float w;
+            route_token(scores + static_cast<int64_t>(tl) * E, E, k, G, vpl, lig, id, w);
+            if (lig < k) {
+                atomicOr(&bits[id * kWords + (tl >> 5)], 1u << (tl & 31));
+                if (tl == me) {
+                    my_ids[lig] = id;
+                    weights[static_cast<int64_t>(me) * k + lig] = from_f32<T>(w);
+                    if (ids_out) ids_out[static_cast<int64_t>(me) * k + lig] = id;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    word_prefix(bits, wordpre, count, E);
+    __syncthreads();
+    if (threadIdx.x == 0) {                    // exclusive scan over experts, in place
+        int run = 0;
+        for (int e = 0; e < E; ++e) {
+            int c = count[e];
+            count[e] = run;
+            run += c;
+        }
+        count[E] = run;
+    }
+    __syncthreads();
+    if (me == 0)
+        for (int e = threadIdx.x; e <= E; e += blockDim.x) off[e] = count[e];
+    if (threadIdx.x < k) {
+        int e = my_ids[threadIdx.x];
+        int64_t pos = count[e] + rank_in_chunk(bits, wordpre, e, me);
+        my_inv[threadIdx.x] = pos;
+        inv[static_cast<int64_t>(me) * k + threadIdx.x] = pos;
+    }
+    __syncthreads();
+    expand_row(X, Xp, static_cast<int64_t>(me), H, k, my_inv, vec);
+}
+
+template <typename T>
+int select_impl(const void *X_, const void *scores_, int64_t Ttok, int64_t H, int E, int k, void *Xp_, void *w_,
+                int64_t *inv, int64_t *off, int32_t *ids, void *ws, hipStream_t s)
+{
+    const T *X = static_cast<const T *>(X_);
+    const T *scores = static_cast<const T *>(scores_);
+    T *Xp = static_cast<T *>(Xp_);
+    T *w = static_cast<T *>(w_);
+    int G = 8;
+    while (G < E && G < kWave) G <<= 1;
+    const int vpl = (E + G - 1) / G;
+    const bool vec = (H * sizeof(T)) % 16 == 0 && aligned16(X) && aligned16(Xp);
+    const int64_t R = Ttok * k;
+
+    if (Ttok == 0) {   // offsets are all zero; nothing else to write
+        select_scan_kernel<<<1, 256, 0, s>>>(nullptr, 0, E, 0, off);
+        OPMX_LAUNCH_CHECK();
+        return OPMX_OK;
+    }
+    if (Ttok <= kChunk && Ttok * G <= kChunk * 8) {
+        select_small_kernel<T><<<static_cast<unsigned>(Ttok), kChunk, 0, s>>>(
+            X, scores, static_cast<int>(Ttok), H, E, k, G, vpl, Xp, w, inv, off, ids, vec);
+        OPMX_LAUNCH_CHECK();
+        return OPMX_OK;
+    }
+    const int nchunks = static_cast<int>(ceil_div(Ttok, kChunk));
+    char *wsb = static_cast<char *>(ws);
+    int32_t *hist = reinterpret_cast<int32_t *>(wsb);
+    int32_t *idbuf = ids ? ids : reinterpret_cast<int32_t *>(wsb + ceil_div(sizeof(int32_t) * nchunks * E, 256) * 256);
+    select_topk_kernel<T><<<nchunks, kChunk, 0, s>>>(scores, Ttok, E, k, G, vpl, w, idbuf, hist);
+    OPMX_LAUNCH_CHECK();
+    select_scan_kernel<<<1, 256, 0, s>>>(hist, nchunks, E, R, off);
+    OPMX_LAUNCH_CHECK();
+    select_rank_kernel<<<nchunks, kChunk, 0, s>>>(idbuf, hist, off, Ttok, E, k, inv);
+    OPMX_LAUNCH_CHECK();
+    const unsigned grid = static_cast<unsigned>(Ttok < 65536 ? Ttok : 65536);
+    select_expand_kernel<T><<<grid, 256, 0, s>>>(X, Xp, inv, Ttok, H, k, vec);
+    OPMX_LAUNCH_CHECK();
+    return OPMX_OK;
+}
+
+}  // namespace
+
+size_t moe_select_workspace_bytes(int64_t T, int E, int k)
+{
+    if (T <= 0) return 256;
+    const int64_t nchunks = ceil_div(T, kChunk);
+    return static_cast<size_t>(ceil_div(sizeof(int32_t) * nchunks * E, 256) * 256 +
+                               ceil_div(sizeof(int32_t) * T * k, 256) * 256);
+}
+
+int launch_moe_select(const void *X, const void *scores, int64_t T, int64_t H, int E, int k, int dtype,
+                      void *Xp, void *w, int64_t *inv, int64_t *off, int32_t *ids, void *ws, hipStream_t s)
+{
+    switch (dtype) {
+        case OPMX_DTYPE_F32: return select_impl<float>(X, scores, T, H, E, k, Xp, w, inv, off, ids, ws, s);
+        case OPMX_DTYPE_F16: return select_impl<f16>(X, scores, T, H, E, k, Xp, w, inv, off, ids, ws, s);
+        case OPMX_DTYPE_BF16: return select_impl<bf16>(X, scores, T, H, E, k, Xp, w, inv, off, ids, ws, s);
+    }
+    return OPMX_ERR_UNSUPPORTED;
+}
+
+}  // namespace opmx

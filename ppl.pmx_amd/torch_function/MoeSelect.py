@@ -1,0 +1,58 @@
+"""``opmx::MoeSelect`` on MI355X.
+
+Drop-in for ``torch_function/MoeSelect.py`` of OpenPPL/ppl.pmx: same positional
+signature, same ONNX node, same eager results (``MoeSelect.py:37-64``) with the
+tie rule fixed to "lower expert id first".  The eager branch is one call into
+``opmx_moe_select``.
+"""
+import torch
+
+from . import _lib
+
+
+class MoeSelect(torch.autograd.Function):
+    @staticmethod
+    def symbolic(g, X, scores, num_experts, num_experts_per_token):
+        # node layout of MoeSelect.py:5-17: two inputs, two int attributes, four outputs
+        outs = g.op("opmx::MoeSelect", X, scores, outputs=4,
+                    num_experts_i=num_experts, num_experts_per_token_i=num_experts_per_token)
+        return tuple(outs)
+
+    @staticmethod
+    def forward(ctx, X, scores, num_experts, num_experts_per_token):
+        E, k = int(num_experts), int(num_experts_per_token)
+        lead, H = tuple(X.shape[:-1]), X.shape[-1]
+        if torch.onnx.is_in_onnx_export():
+            # shape/dtype placeholders, returned in the eager (documented) order
+            z = lambda *shape, dtype: torch.zeros(*shape, dtype=dtype, device=X.device)
+            return (z(*lead, k, H, dtype=X.dtype), z(*lead, k, dtype=X.dtype),
+                    z(*lead, k, dtype=torch.int64), z(E + 1, dtype=torch.int64))
+
+        dev = _lib.require_gpu("moe_select", X, scores)
+        if scores.shape[-1] != E or tuple(scores.shape[:-1]) != lead:
+            raise ValueError("moe_select: scores shape {} does not match X {} / num_experts {}".format(
+                tuple(scores.shape), tuple(X.shape), E))
+        if scores.dtype != X.dtype:
+            raise TypeError("moe_select: X and scores must share one dtype")
+        if not (1 <= k <= E):
+            raise ValueError("moe_select: need 1 <= num_experts_per_token <= num_experts")
+        dt = _lib.dtype_id(X, "moe_select")
+        Xf = X.reshape(-1, H).contiguous()
+        sf = scores.reshape(-1, E).contiguous()
+        T = Xf.shape[0]
+        x_expand = torch.empty(T * k, H, dtype=X.dtype, device=dev)
+        weights = torch.empty(T, k, dtype=scores.dtype, device=dev)
+        inv = torch.empty(T * k, dtype=torch.int64, device=dev)
+        off = torch.empty(E + 1, dtype=torch.int64, device=dev)
+        L = _lib.lib()
+        ws = _lib.workspace(L.opmx_moe_select_workspace_bytes(T, E, k), dev)
+        _lib.check(L.opmx_moe_select(_lib.ptr(Xf), _lib.ptr(sf), T, H, E, k, dt, _lib.ptr(x_expand),
+                                     _lib.ptr(weights), _lib.ptr(inv), _lib.ptr(off), None,
+                                     _lib.ptr(ws), ws.numel(), _lib.stream_ptr(dev)), "moe_select")
+        return (x_expand.view(*lead, k, H), weights.view(*lead, k), inv.view(*lead, k), off)
+
+
+def moe_select(X: torch.Tensor, scores: torch.Tensor, num_experts: int, num_experts_per_token: int):
+    """-> (X_expand_permute [*,k,H], expert_weights [*,k], invert_permutation [*,k] i64,
+    expert_offset [E+1] i64)"""
+    return MoeSelect.apply(X, scores, num_experts, num_experts_per_token)

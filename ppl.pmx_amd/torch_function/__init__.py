@@ -1,0 +1,18 @@
+"""MI355X-native implementation of the OPMX mixture-of-experts operators.
+
+Import it the way the reference's consumers import theirs
+(``import torch_function as OPMX`` with this package's parent directory on
+``sys.path``); the seven functions below keep the reference's names and
+positional signatures (``torch_function/__init__.py:15,17-20,37-38`` of
+OpenPPL/ppl.pmx).
+"""
+from .Linear import linear
+from .MoeColumnParallelLinear import moe_column_parallel_linear, moe_column_parallel_linear_swiglu
+from .MoeReduce import moe_reduce
+from .MoeRowParallelLinear import moe_row_parallel_linear
+from .MoeSelect import moe_select
+from .SiLU import silu
+from .SwiGLU import swiglu
+
+__all__ = ["linear", "moe_column_parallel_linear", "moe_column_parallel_linear_swiglu", "moe_reduce",
+           "moe_row_parallel_linear", "moe_select", "silu", "swiglu"]

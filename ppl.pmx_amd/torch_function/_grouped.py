@@ -1,0 +1,60 @@
+"""Shared eager path of the two grouped expert linears (one C-ABI call each)."""
+import torch
+
+from . import _lib
+
+
+def grouped_linear(op, X, expert_offset, W, B, num_experts, epilogue=_lib.EPILOGUE_NONE):
+    """``Y[off[e]:off[e+1]] = X[off[e]:off[e+1]] @ W[e]^T (+ B[e])`` on the GPU.
+
+    ``op`` is "column" or "row".  Output dtype is ``W.dtype`` on ``X.device``
+    (the reference's export branch states that dtype,
+    ``MoeColumnParallelLinear.py:45``; its eager branch follows the process
+    default dtype).  A row-parallel bias is applied per expert segment.
+    """
+    name = "moe_{}_parallel_linear".format(op)
+    dev = _lib.require_gpu(name, X, expert_offset, W, B)
+    E, N, K = W.shape
+    if E != num_experts:
+        raise ValueError("{}: W holds {} experts, num_experts is {}".format(name, E, num_experts))
+    if X.shape[-1] != K:
+        raise ValueError("{}: X has {} features, W expects {}".format(name, X.shape[-1], K))
+    if expert_offset.numel() != E + 1:
+        raise ValueError("{}: expert_offset must have num_experts + 1 entries".format(name))
+    if X.dtype != W.dtype or (B is not None and B.dtype != W.dtype):
+        raise TypeError("{}: X, W and B must share one dtype".format(name))
+    if B is not None and tuple(B.shape) != (E, N):
+        raise ValueError("{}: B must be [num_experts, out_features_per_partition]".format(name))
+    dt = _lib.dtype_id(W, name)
+    Xf = X.reshape(-1, K).contiguous()
+    Wc = W.detach().contiguous()
+    Bc = None if B is None else B.detach().contiguous()
+    off = expert_offset.to(torch.int64).contiguous()
+    R = Xf.shape[0]
+    n_out = N // 2 if epilogue == _lib.EPILOGUE_SWIGLU else N
+    # rows of one expert never exceed the token count when X is [*, k, K] from moe_select
+    hint = R // X.shape[-2] if X.dim() >= 3 and X.shape[-2] > 0 else 0
+    Y = torch.empty(R, n_out, dtype=W.dtype, device=dev)
+    L = _lib.lib()
+    ws = None
+    ws_bytes = 0
+    if epilogue != _lib.EPILOGUE_NONE:
+        ws = _lib.workspace(L.opmx_moe_grouped_gemm_workspace_bytes(E, R, K, N, dt), dev)
+        ws_bytes = ws.numel()
+    if op == "column":
+        rc = L.opmx_moe_column_parallel_linear(_lib.ptr(Xf), _lib.ptr(off), _lib.ptr(Wc), _lib.ptr(Bc), E, R, K, N,
+                                               dt, epilogue, hint, _lib.ptr(Y), _lib.ptr(ws), ws_bytes,
+                                               _lib.stream_ptr(dev))
+    else:
+        rc = L.opmx_moe_row_parallel_linear(_lib.ptr(Xf), _lib.ptr(off), _lib.ptr(Wc), _lib.ptr(Bc), E, R, K, N,
+                                            dt, hint, _lib.ptr(Y), _lib.ptr(ws), ws_bytes, _lib.stream_ptr(dev))
+    _lib.check(rc, name)
+    return Y.view(*X.shape[:-1], n_out)
+
+
+def linear_attrs(num_experts, in_features, out_features, has_bias, **extra):
+    """Attribute set shared by the two ``opmx::Moe*ParallelLinear`` nodes."""
+    attrs = dict(num_experts_i=num_experts, in_features_i=in_features, out_features_i=out_features,
+                 bias_term_i=bool(has_bias))
+    attrs.update(extra)
+    return attrs

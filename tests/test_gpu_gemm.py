@@ -1,0 +1,150 @@
+"""GPU parity: grouped expert GEMMs (generic, MFMA-tiled and weight-streaming
+kernels, bias, SwiGLU epilogue, ragged / empty / partial offsets) against the CPU
+oracle on identical inputs.  Tolerance: 2 ulp of the output dtype (one rounding
+plus fp32 accumulation order), relative to max(|ref|, 2% of max|ref|)."""
+import os
+
+import pytest
+import torch
+
+from _util import assert_close_ulp, dev
+from oracle import moe_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def opmx():
+    import torch_function as OPMX
+    return OPMX
+
+
+def offsets(sizes):
+    return torch.tensor([0] + list(torch.tensor(sizes).cumsum(0).tolist()), dtype=torch.int64)
+
+
+def run_case(kind, sizes, K, N, dtype, bias, env=None, swiglu=False, lead3=False, off=None, R=None, seed=0):
+    """kind: 'column' | 'row'.  sizes: rows per expert."""
+    OPMX = opmx()
+    E = len(sizes)
+    off = offsets(sizes) if off is None else off
+    R = int(sum(sizes)) if R is None else R
+    g = torch.Generator().manual_seed(seed + K + N + R)
+    X = torch.randn(R, K, generator=g).to(dtype)
+    W = (torch.randn(E, N, K, generator=g) * 0.05).to(dtype)
+    B = torch.randn(E, N, generator=g).to(dtype) if bias else None
+    if lead3:                                  # [T, k, K] as MoeSelect returns it
+        X = X.view(R // 2, 2, K)
+    old = {}
+    for key, val in (env or {}).items():
+        old[key] = os.environ.get(key)
+        os.environ[key] = val
+    try:
+        args = (X.to(dev()), off.to(dev()), W.to(dev()), None if B is None else B.to(dev()))
+        if swiglu:
+            Y = OPMX.moe_column_parallel_linear_swiglu(*args, E, K, N)
+        elif kind == "column":
+            Y = OPMX.moe_column_parallel_linear(*args, None, E, K, N, False)
+        else:
+            Y = OPMX.moe_row_parallel_linear(*args, None, E, K, N, True)
+        torch.cuda.synchronize()
+    finally:
+        for key, val in old.items():
+            if val is None:
+                os.environ.pop(key, None)
+            else:
+                os.environ[key] = val
+    ref = O.moe_column_parallel_linear(X, off, W, B, acc=torch.float64, out_dtype=torch.float64)
+    if swiglu:
+        ref = O.swiglu(ref, acc=torch.float64)
+    assert Y.dtype == dtype and Y.shape == ref.shape
+    f32 = dtype == torch.float32
+    assert_close_ulp(Y, ref, dtype, ulps=64 if f32 else 2, floor=0.25 if f32 else 0.02,
+                     what="{} {} K{} N{} {} {}".format(kind, sizes, K, N, dtype, env))
+    return Y
+
+
+RAGGED8 = [5, 0, 17, 1, 0, 64, 3, 38]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("swiglu", [False, True])
+def test_generic_kernel(dtype, swiglu):
+    env = {"OPMX_MOE_GEMM": "generic"}
+    run_case("column", RAGGED8, 72, 100, dtype, True, env, swiglu=swiglu)
+    run_case("row", [3, 130, 0, 70], 50, 66, dtype, False, env, swiglu=swiglu)
+    run_case("column", [1], 8, 2, dtype, True, env, swiglu=swiglu)
+
+
+def test_tiny_config_fp32_shapes():
+    """The CPU-runnable reference config: H=1024, I=2816, E=8, fp32."""
+    sizes = [20, 9, 31, 0, 16, 25, 12, 15]
+    run_case("column", sizes, 1024, 5632, torch.float32, False)
+    run_case("row", sizes, 2816, 1024, torch.float32, False)
+    run_case("column", sizes, 1024, 5632, torch.float32, True, swiglu=True)
+
+
+@pytest.mark.parametrize("variant", ["0", "1", "2", "3"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_tiled_kernel_variants(variant, dtype):
+    env = {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": variant}
+    sizes = [300, 0, 129, 1, 256, 77, 0, 513]
+    run_case("column", sizes, 256, 512, dtype, False, env)
+    run_case("row", sizes, 448, 384, dtype, True, env)
+    run_case("column", sizes, 128, 200, dtype, True, env)                 # N not a tile multiple
+    run_case("column", sizes, 192, 512, dtype, True, env, swiglu=True)
+    run_case("column", sizes, 64, 1000, dtype, False, env, swiglu=True)   # D=500: ragged epilogue tile
+
+
+@pytest.mark.parametrize("variant", ["0", "1"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_stream_kernel_variants(variant, dtype):
+    env = {"OPMX_MOE_GEMM": "stream", "OPMX_MOE_GEMM_STREAM_VARIANT": variant}
+    for sizes in ([1, 0, 1, 0, 0, 0, 0, 0],               # T=1 decode: two active experts
+                  [8, 9, 7, 11, 0, 16, 5, 8],             # <= 16 rows per expert
+                  [30, 2, 17, 0, 32, 1, 25, 21],          # <= 32
+                  [64, 40, 0, 3, 50, 33, 1, 65],          # <= 64 (+ one expert with a second tile)
+                  [128, 0, 0, 100, 7, 0, 0, 21]):
+        run_case("column", sizes, 512, 192, dtype, False, env, lead3=False)
+        run_case("row", sizes, 1408, 128, dtype, True, env)           # K not a multiple of the K-chunk
+    run_case("column", [8, 9, 7, 11, 0, 16, 5, 8], 256, 100, dtype, True, env)      # N not a multiple of 64
+    run_case("column", [8, 9, 7, 11, 0, 16, 5, 8], 264, 128, dtype, True, env)      # K % 8 == 0 only
+    run_case("column", [8, 9, 7, 11, 0, 16, 5, 8], 512, 256, dtype, True, env, swiglu=True)
+    run_case("column", [4] * 64, 256, 128, dtype, False, env)                       # 64 experts
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_automatic_selection_and_hint(dtype):
+    # [T, k, K] input: the wrapper passes rows-per-expert hint T
+    run_case("column", [10, 6, 0, 16, 8, 8, 9, 7], 512, 256, dtype, False, lead3=True)
+    run_case("column", [700, 6, 0, 16, 800, 8, 90, 428], 512, 256, dtype, False, lead3=True)
+    run_case("row", [700, 6, 0, 16, 800, 8, 90, 428], 512, 256, dtype, True)
+
+
+@pytest.mark.parametrize("force", ["generic", "tiled", "stream"])
+def test_rows_owned_by_no_expert_are_zero(force):
+    """off = arange(E+1) with more rows than experts is the reference's own demo
+    input (MoeColumnParallelLinear.py:135-136): row e uses expert e, the rest stay 0.
+    Also offsets that start after row 0."""
+    E, K, N = 8, 128, 192
+    env = {"OPMX_MOE_GEMM": force}
+    Y = run_case("column", [1] * E, K, N, torch.float16, True, env, off=torch.arange(E + 1), R=80)
+    assert torch.count_nonzero(Y[E:]) == 0
+    off = torch.tensor([5, 5, 9, 20, 20, 31, 40, 41, 60])
+    Y = run_case("row", [0] * E, K, N, torch.float16, False, env, off=off, R=64)
+    assert torch.count_nonzero(Y[:5]) == 0 and torch.count_nonzero(Y[60:]) == 0
+
+
+def test_argument_errors():
+    OPMX = opmx()
+    d = dev()
+    X = torch.zeros(4, 2, 64, device=d, dtype=torch.float16)
+    off = torch.tensor([0, 8], device=d)
+    W = torch.zeros(1, 32, 64, device=d, dtype=torch.float16)
+    with pytest.raises(AssertionError):                       # MoeColumnParallelLinear.py:40
+        OPMX.moe_column_parallel_linear(X, off, W, None, None, 1, 63, 32, False)
+    with pytest.raises(TypeError):
+        OPMX.moe_column_parallel_linear(X.float(), off, W, None, None, 1, 64, 32, False)
+    with pytest.raises(RuntimeError):
+        OPMX.moe_row_parallel_linear(X.cpu(), off.cpu(), W.cpu(), None, None, 1, 64, 32, True)
+    Y = OPMX.moe_row_parallel_linear(X[:0], torch.zeros(2, dtype=torch.int64, device=d), W, None, None, 1, 64, 32)
+    assert Y.shape == (0, 2, 32)

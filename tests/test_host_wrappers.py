@@ -1,0 +1,121 @@
+"""CPU checks of the host-side mirror of the reference interface: names and
+signatures, ONNX symbolics (node type, input order, attribute names and values
+as in the reference's symbolic() functions), export placeholders, and the "no
+CPU fallback" rule."""
+import contextlib
+import inspect
+import io
+import re
+import warnings
+
+import pytest
+import torch
+
+import torch_function as OPMX
+from model_zoo.mixtral.modeling.dynamic_batching.Model import MoeFeedForward
+
+
+def test_public_names_and_signatures():
+    # torch_function/__init__.py:15,17-20,37-38 and the wrapper defs of each file
+    sig = lambda f: list(inspect.signature(f).parameters)
+    assert sig(OPMX.moe_select) == ["X", "scores", "num_experts", "num_experts_per_token"]
+    assert sig(OPMX.moe_reduce) == ["Y", "expert_weights", "invert_permutation", "num_experts_per_token"]
+    assert sig(OPMX.moe_column_parallel_linear) == ["X", "expert_offset", "W", "B", "proc_group", "num_experts",
+                                                    "in_features", "out_features", "gather_output"]
+    assert sig(OPMX.moe_row_parallel_linear) == ["X", "expert_offset", "W", "B", "proc_group", "num_experts",
+                                                 "in_features", "out_features", "input_is_parallel"]
+    assert sig(OPMX.swiglu) == ["X", "beta"] and sig(OPMX.silu) == ["X", "gate"]
+    assert sig(OPMX.linear) == ["X", "W", "B", "in_features", "out_features"]
+    p = inspect.signature(OPMX.moe_column_parallel_linear).parameters
+    assert p["gather_output"].default is True
+    assert inspect.signature(OPMX.moe_row_parallel_linear).parameters["input_is_parallel"].default is False
+
+
+def test_no_cpu_fallback():
+    x = torch.randn(4, 16)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        OPMX.moe_select(x, torch.randn(4, 8), 8, 2)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        OPMX.swiglu(x)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        OPMX.moe_reduce(torch.randn(4, 2, 8), torch.rand(4, 2), torch.arange(8).view(4, 2), 2)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        OPMX.linear(x, torch.randn(8, 16), None, 16, 8)
+    with pytest.raises(AssertionError):          # the reference's in_features assert comes first
+        OPMX.moe_column_parallel_linear(x, torch.arange(3), torch.randn(2, 8, 16), None, None, 2, 15, 8, False)
+
+
+def export_graph(mod, args):
+    """TorchScript-exporter graph of `mod` at opset 11 (what torch.onnx.export
+    builds before serialising; the `onnx` package is not needed for this)."""
+    from torch.onnx._internal.torchscript_exporter import utils as U
+    from torch.onnx._internal.torchscript_exporter._globals import GLOBALS
+    GLOBALS.export_onnx_opset_version = 11
+    with warnings.catch_warnings(), contextlib.redirect_stdout(io.StringIO()):
+        warnings.simplefilter("ignore")
+        with U.exporter_context(mod, torch.onnx.TrainingMode.EVAL, False):
+            GLOBALS.in_onnx_export = True
+            try:
+                graph, _, out = U._model_to_graph(mod, args)
+            finally:
+                GLOBALS.in_onnx_export = False
+    return graph, out
+
+
+def nodes_of(graph):
+    found = []
+    for n in graph.nodes():
+        if n.kind().startswith("opmx::"):
+            attrs = {a: (n.f(a) if n.kindOf(a) == "f" else n.i(a)) for a in n.attributeNames()}
+            found.append((n.kind(), len(list(n.inputs())), len(list(n.outputs())), attrs))
+    return found
+
+
+@pytest.mark.parametrize("fused,bias", [(True, False), (False, True)])
+def test_mixtral_block_exports_reference_nodes(fused, bias):
+    H, I, E, k = 64, 96, 8, 2
+    m = MoeFeedForward(MoeFeedForward.params(H, I, E, k), 0, fused, bias, None, fuse_swiglu_epilogue=True)
+    graph, out = export_graph(m, (torch.randn(5, H),))
+    got = nodes_of(graph)
+    nb = 1 if bias else 0
+    col = lambda n: ("opmx::MoeColumnParallelLinear", 3 + nb, 1,
+                     dict(num_experts=E, in_features=H, out_features=n, bias_term=nb, gather_output=0))
+    want = [("opmx::Linear", 2, 1, dict(in_features=H, out_features=E, bias_term=0)),
+            ("opmx::MoeSelect", 2, 4, dict(num_experts=E, num_experts_per_token=k))]
+    if fused:
+        want += [col(2 * I), ("opmx::SwiGLU", 1, 1, dict(beta=1.0))]
+    else:
+        want += [col(I), col(I), ("opmx::SiLU", 2, 1, {})]
+    want += [("opmx::MoeRowParallelLinear", 3 + nb, 1,
+              dict(num_experts=E, in_features=I, out_features=H, bias_term=nb, input_is_parallel=1)),
+             ("opmx::MoeReduce", 3, 1, dict(num_experts_per_token=k))]
+    assert got == want
+    assert tuple(out.shape) == (5, H)
+
+
+def test_export_placeholders_have_eager_order_and_types():
+    class Sel(torch.nn.Module):
+        def forward(self, x, s):
+            return OPMX.moe_select(x, s, 8, 2)
+    graph, out = export_graph(Sel(), (torch.randn(3, 4, 16).half(), torch.randn(3, 4, 8).half()))
+    xe, w, inv, off = out
+    assert xe.shape == (3, 4, 2, 16) and xe.dtype == torch.float16
+    assert w.shape == (3, 4, 2) and w.dtype == torch.float16
+    assert inv.shape == (3, 4, 2) and inv.dtype == torch.int64
+    assert off.shape == (9,) and off.dtype == torch.int64
+    text = str(graph)
+    assert re.search(r"Half\(.*\), %\d+ : Half\(.*\), %\d+ : Long\(.*\), %\d+ : Long\(.*\) = opmx::MoeSelect", text)
+
+
+def test_tensor_parallel_is_refused():
+    class FakeGroup:
+        def size(self):
+            return 2
+    import unittest.mock as mock
+    with mock.patch("torch.distributed.get_world_size", return_value=2):
+        with pytest.raises(NotImplementedError):
+            OPMX.moe_row_parallel_linear(torch.randn(4, 16), torch.arange(3), torch.randn(2, 8, 16), None,
+                                         FakeGroup(), 2, 16, 8, True)
+        with pytest.raises(NotImplementedError):
+            OPMX.moe_column_parallel_linear(torch.randn(4, 16), torch.arange(3), torch.randn(2, 8, 16), None,
+                                            FakeGroup(), 2, 16, 8, False)
