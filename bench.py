@@ -1,0 +1,219 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE layer hot path on one MI355X.
+
+A "step" is one forward pass of the Mixtral-style MoE layer (router gate ->
+MoeSelect -> gate/up grouped GEMM -> SwiGLU -> down grouped GEMM -> MoeReduce)
+through the drop-in operators, over one batch of synthetic tokens that is
+already resident in HBM.  Prints ONE JSON line:
+
+  value / ms_per_step  whole-layer tokens/s and latency over exactly --steps steps
+  roofline             the dominant kernel (gate/up grouped GEMM): algorithmic bytes
+                       or flops per launch / mean launch duration (HIP events on
+                       the launch stream, taken inside the timed steps) vs MI355X peak
+  layer                the same accounting for the whole layer
+  per_op_us            mean duration of each operator (separate untimed pass)
+  cpu_baseline         the CPU oracle (PyTorch CPU restatement of the reference
+                       operator sequence) on the host cores, bounded sample
+
+Workloads (--workload): decode-T{1,8,32,128} and prefill-T{2048,8192} at the
+Mixtral-8x7B shape (fp16), fine-T{32,4096} (64 experts, top-8, bf16),
+8x22b-T{16,4096}.  Default: decode-T32, the configuration the metric is quoted on.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "ppl.pmx_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, vendor figure
+MFMA_PEAK_TFLOPS = 2500.0      # dense fp16/bf16 MFMA, vendor figure
+
+SHAPES = {
+    "decode": dict(H=4096, E=8, k=2, I=14336, dtype="float16", skew=0.0, name="mixtral-8x7b"),
+    "prefill": dict(H=4096, E=8, k=2, I=14336, dtype="float16", skew=4.0, name="mixtral-8x7b"),
+    "fine": dict(H=2048, E=64, k=8, I=1408, dtype="bfloat16", skew=0.0, name="fine-grained-64x8"),
+    "8x22b": dict(H=6144, E=8, k=2, I=16384, dtype="float16", skew=0.0, name="mixtral-8x22b-shape"),
+}
+
+
+def parse_workload(w):
+    kind, t = w.split("-T")
+    cfg = dict(SHAPES[kind])
+    cfg["T"] = int(t)
+    cfg["kind"] = kind
+    return cfg
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="decode-T32")
+    ap.add_argument("--fuse-swiglu", action="store_true", help="apply SwiGLU in the gate/up GEMM epilogue")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (TP=1, no collectives); --gpus {} is not "
+                 "supported, run with --gpus 1".format(args.gpus))
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs an MI355X (no GPU visible)")
+    import torch_function as OPMX
+    from model_zoo.mixtral.modeling.dynamic_batching.Model import MoeFeedForward
+
+    cfg = parse_workload(args.workload)
+    T, H, E, k, I = cfg["T"], cfg["H"], cfg["E"], cfg["k"], cfg["I"]
+    dtype = getattr(torch, cfg["dtype"])
+    s = 2
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    # ---- synthetic inputs, seeded, drawn on the device (x~N(0,1), weights~N(0,0.02))
+    g = torch.Generator(device="cuda").manual_seed(0)
+    x = torch.randn(T, H, generator=g, device=dev).to(dtype)
+    layer = MoeFeedForward(MoeFeedForward.params(H, I, E, k), 0, True, False, None, dtype=dtype, device=dev,
+                           fuse_swiglu_epilogue=args.fuse_swiglu)
+    layer.gate.weight.data = (torch.randn(E, H, generator=g, device=dev) * 0.02).to(dtype)
+    for e in range(E):
+        layer.wu.weight.data[e] = (torch.randn(2 * I, H, generator=g, device=dev) * 0.02).to(dtype)
+        layer.w2.weight.data[e] = (torch.randn(H, I, generator=g, device=dev) * 0.02).to(dtype)
+    if cfg["skew"] > 0:       # Zipf(s=1.2) per-expert logit bias: skewed expert load
+        p = torch.arange(1, E + 1, dtype=torch.float64) ** -1.2
+        bias = (cfg["skew"] * torch.log(p / p.sum())).to(dtype).to(dev)
+        layer.gate.bias = torch.nn.Parameter(bias, requires_grad=False)
+    Wg, wu, w2, gb = layer.gate.weight, layer.wu.weight, layer.w2.weight, layer.gate.bias
+
+    # ---- one instrumented pass: routing statistics + per-operator durations
+    def ops(record=None):
+        def timed(name, fn):
+            if record is None:
+                return fn()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            r = fn()
+            b.record()
+            record.append((name, a, b))
+            return r
+        sc = timed("router_linear", lambda: OPMX.linear(x, Wg, gb, H, E))
+        xe, w, inv, off = timed("moe_select", lambda: OPMX.moe_select(x, sc, E, k))
+        if args.fuse_swiglu:
+            act = timed("gate_up_gemm", lambda: OPMX.moe_column_parallel_linear_swiglu(xe, off, wu, None, E, H, 2 * I))
+        else:
+            h = timed("gate_up_gemm", lambda: OPMX.moe_column_parallel_linear(xe, off, wu, None, None, E, H, 2 * I, False))
+            act = timed("swiglu", lambda: OPMX.swiglu(h))
+        y = timed("down_gemm", lambda: OPMX.moe_row_parallel_linear(act, off, w2, None, None, E, I, H, True))
+        out = timed("moe_reduce", lambda: OPMX.moe_reduce(y, w, inv, k))
+        return out, off
+
+    with torch.inference_mode():
+        for _ in range(max(args.warmup, 1)):
+            out, off = ops()
+        torch.cuda.synchronize()
+        counts = (off[1:] - off[:-1]).cpu()
+        active = int((counts > 0).sum())
+        R = T * k
+        if cfg["kind"] == "prefill":
+            assert float(counts.max()) / R > 0.40, "skewed-routing config needs the largest expert above 40%"
+
+        # ---- timed region: exactly --steps steps; HIP events bracket the dominant kernel
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        gemm1 = (lambda xe, off: OPMX.moe_column_parallel_linear_swiglu(xe, off, wu, None, E, H, 2 * I)) \
+            if args.fuse_swiglu else \
+            (lambda xe, off: OPMX.moe_column_parallel_linear(xe, off, wu, None, None, E, H, 2 * I, False))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            sc = OPMX.linear(x, Wg, gb, H, E)
+            xe, w, inv, off = OPMX.moe_select(x, sc, E, k)
+            ev[i][0].record()
+            h = gemm1(xe, off)
+            ev[i][1].record()
+            act = h if args.fuse_swiglu else OPMX.swiglu(h)
+            y = OPMX.moe_row_parallel_linear(act, off, w2, None, None, E, I, H, True)
+            out = OPMX.moe_reduce(y, w, inv, k)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        ms_per_step = dt / args.steps * 1e3
+        gemm1_ms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
+
+        # ---- per-operator durations (untimed extra pass, averaged)
+        per_op = {}
+        reps = 20
+        for _ in range(reps):
+            rec = []
+            ops(rec)
+            torch.cuda.synchronize()
+            for name, a, b in rec:
+                per_op[name] = per_op.get(name, 0.0) + a.elapsed_time(b) * 1e3 / reps
+
+    # ---- algorithmic work
+    w_bytes_gemm1 = active * 2 * I * H * s
+    w_bytes_gemm2 = active * H * I * s
+    n1 = I if args.fuse_swiglu else 2 * I
+    gemm1_bytes = w_bytes_gemm1 + R * H * s + R * n1 * s
+    gemm1_flops = 2.0 * R * H * 2 * I
+    layer_bytes = w_bytes_gemm1 + w_bytes_gemm2 + 2 * T * H * s + E * H * s
+    layer_flops = T * (k * (2.0 * H * 2 * I + 2.0 * I * H) + 2.0 * H * E)
+    hbm_bound = (layer_flops / layer_bytes) < (MFMA_PEAK_TFLOPS * 1e12) / (HBM_PEAK_GBS * 1e9)
+    if hbm_bound:
+        ach = gemm1_bytes / (gemm1_ms * 1e-3) / 1e9
+        roof = dict(bound="hbm", kernel="gate_up_grouped_gemm", achieved=round(ach, 1), peak=HBM_PEAK_GBS,
+                    unit="GB/s", frac=round(ach / HBM_PEAK_GBS, 4), traffic=None,
+                    algorithmic_bytes=int(gemm1_bytes), launch_ms=round(gemm1_ms, 4))
+        lach = layer_bytes / (ms_per_step * 1e-3) / 1e9
+        lay = dict(bound="hbm", achieved=round(lach, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+                   frac=round(lach / HBM_PEAK_GBS, 4), algorithmic_bytes=int(layer_bytes))
+    else:
+        ach = gemm1_flops / (gemm1_ms * 1e-3) / 1e12
+        roof = dict(bound="mfma", kernel="gate_up_grouped_gemm", achieved=round(ach, 1), peak=MFMA_PEAK_TFLOPS,
+                    unit="TFLOP/s", frac=round(ach / MFMA_PEAK_TFLOPS, 4), traffic=None,
+                    algorithmic_flops=int(gemm1_flops), launch_ms=round(gemm1_ms, 4))
+        lach = layer_flops / (ms_per_step * 1e-3) / 1e12
+        lay = dict(bound="mfma", achieved=round(lach, 1), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
+                   frac=round(lach / MFMA_PEAK_TFLOPS, 4), algorithmic_flops=int(layer_flops))
+
+    result = {
+        "metric": "MoE-layer tokens/sec at Mixtral-8x7B shape, fp16, 1 GPU; % HBM/MFMA roofline",
+        "value": round(T / (ms_per_step * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": {"float16": "f16", "bfloat16": "bf16"}[cfg["dtype"]], "data": "synthetic",
+        "config": {"workload": "{} MoE layer {}, T={} tokens, hidden={}, experts={}, top-{}, ffn={}, TP=1".format(
+            cfg["name"], "decode" if hbm_bound else "prefill", T, H, E, k, I),
+            "path": "drop-in operator sequence" + (" + fused SwiGLU epilogue" if args.fuse_swiglu else ""),
+            "active_experts": active, "max_expert_share": round(float(counts.max()) / R, 3)},
+        "roofline": roof, "layer": lay, "per_op_us": {n: round(v, 1) for n, v in per_op.items()},
+        "device": torch.cuda.get_device_name(0), "cu_count": torch.cuda.get_device_properties(0).multi_processor_count,
+    }
+
+    # ---- CPU baseline: the oracle (PyTorch CPU restatement of the reference operator
+    # sequence) on this box's host cores.  Checker code, timed only here.
+    if not args.no_cpu_baseline:
+        from oracle import moe_oracle as O
+        Tc = T if T <= 512 else 512            # bounded sample of the same workload
+        xc, Wgc, wuc, w2c = x[:Tc].cpu(), Wg.cpu(), wu.cpu(), w2.cpu()
+        gbc = None if gb is None else gb.cpu()
+        runs, spent = 0, 0.0
+        while runs < 1 or (spent < args.cpu_seconds and runs < 20):
+            c0 = time.perf_counter()
+            O.moe_layer(xc, Wgc, wuc, w2c, E, k, router_bias=gbc, round_between_ops=True)
+            spent += time.perf_counter() - c0
+            runs += 1
+        result["cpu_baseline"] = {
+            "value": round(Tc / (spent / runs), 2), "unit": "tokens/s", "cores": torch.get_num_threads(),
+            "kind": "port", "host_cpus": os.cpu_count(),
+            "sample": "{} run(s) of the same layer on the first {} tokens, fp32 accumulation on {} inputs, "
+                      "{:.1f} s of CPU time".format(runs, Tc, cfg["dtype"], spent)}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
