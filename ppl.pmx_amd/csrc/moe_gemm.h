@@ -9,6 +9,7 @@ namespace opmx {
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // a 16-byte register quad
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
 template <typename T> struct Mfma;
@@ -64,10 +65,12 @@ __device__ __forceinline__ MTile find_mtile(const int64_t *__restrict__ off, int
         if (hi < lo) hi = lo;
         const int64_t nt = (hi - lo + BM - 1) / BM;
         if (tile < nt) {
-            t.e = e;
-            t.row0 = lo + tile * BM;
-            const int64_t left = hi - t.row0;
-            t.rows = static_cast<int>(left < BM ? left : BM);
+            // block-uniform by construction; say so to the compiler (scalar registers)
+            const int64_t row0 = lo + tile * BM, left = hi - row0;
+            t.e = __builtin_amdgcn_readfirstlane(e);
+            t.row0 = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0 >> 32))) << 32) |
+                     static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0)));
+            t.rows = __builtin_amdgcn_readfirstlane(static_cast<int>(left < BM ? left : BM));
             return t;
         }
         tile -= nt;

@@ -7,8 +7,9 @@
 //  * a block = 4 waves = 64 consecutive rows of W[e] (one 16-row group per wave)
 //    x one row tile (<= 16*MT rows) of expert e, over the whole K;
 //  * W is fetched with fully coalesced 16-byte loads (a wave instruction reads
-//    1 KiB contiguous), one K-chunk ahead in registers, then transposed into the
-//    MFMA operand layout through a wave-private LDS strip (no block barrier);
+//    1 KiB contiguous) into registers, DEPTH K-chunks ahead, then transposed
+//    into the MFMA operand layout through a wave-private LDS strip (no block
+//    barrier for W);
 //  * the X chunk is shared by the four waves through double-buffered LDS: one
 //    barrier per K-chunk;
 //  * experts with no rows produce no work, so their weights are never touched.
@@ -22,7 +23,13 @@ namespace {
 constexpr int SW = 4;            // waves per block
 constexpr int SROWS = 16 * SW;   // W rows per block
 
-template <typename T, int MT, int KC>
+template <bool NT> __device__ __forceinline__ u32x4 ld16(const char *p)
+{
+    if (NT) return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+    return *reinterpret_cast<const u32x4 *>(p);
+}
+
+template <typename T, int MT, int KC, int DEPTH, bool NT>
 __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restrict__ X,
                                                                const int64_t *__restrict__ off,
                                                                const T *__restrict__ W,
@@ -38,6 +45,7 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
     constexpr int WSTRIP = 16 * RS;
     constexpr int XBUF = XM * RS;
     static_assert(XM * CPR % (SW * 64) == 0, "X chunk must divide over the block");
+    static_assert(DEPTH == 1 || DEPTH == 2, "one or two chunks in flight");
     using frag = typename Mfma<T>::frag;
 
     extern __shared__ __attribute__((aligned(16))) char smem[];   // [SW][WSTRIP] | [2][XBUF]
@@ -51,29 +59,30 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
     char *wstrip = smem + wave * WSTRIP;
     char *xbuf = smem + SW * WSTRIP;
 
-    // ---- this wave's 16 rows of W[e]; rows past N are clamped (masked at the store)
+    // ---- this wave's 16 rows of W[e]: uniform base + per-lane byte offsets.
+    // Rows past N are clamped to row N-1 (their results are masked at the store).
     const int64_t nbase = static_cast<int64_t>(blockIdx.x) * SROWS + wave * 16;
-    const T *We = W + static_cast<int64_t>(mt.e) * N * K;
+    const char *wb = reinterpret_cast<const char *>(W + static_cast<int64_t>(mt.e) * N * K);
+    const char *xb = reinterpret_cast<const char *>(X + mt.row0 * K);
     const int wl_row = lane / (64 / RPL);               // row inside one wave load
     const int wl_k = (lane % (64 / RPL)) * 8;           // k offset inside the chunk
-    const T *wsrc[NLW];
+    uint32_t wrow[NLW];                                 // byte offset of the row start
     int wdst[NLW];
 #pragma unroll
     for (int i = 0; i < NLW; ++i) {
         const int row = i * RPL + wl_row;
         int64_t n = nbase + row;
         n = n < N ? n : N - 1;
-        wsrc[i] = We + n * K + wl_k;
+        wrow[i] = static_cast<uint32_t>(n * K * 2);
         wdst[i] = row * RS + wl_k * 2;
     }
-    // ---- this thread's share of the X chunk
-    const T *xsrc[NLX];
+    uint32_t xrow[NLX];
     int xdst[NLX], xk[NLX];
 #pragma unroll
     for (int i = 0; i < NLX; ++i) {
         const int q = tid + SW * 64 * i, row = q / CPR, c = q % CPR;
         const int r = row < mt.rows ? row : mt.rows - 1;
-        xsrc[i] = X + (mt.row0 + r) * K + c * 8;
+        xrow[i] = static_cast<uint32_t>(r * K * 2);
         xdst[i] = row * RS + c * 16;
         xk[i] = c * 8;
     }
@@ -82,41 +91,71 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
 #pragma unroll
     for (int m = 0; m < MT; ++m) acc[m] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
-    uint4 wreg[NLW], xreg[NLX];
-    auto fetch = [&](int64_t k0) {
-#pragma unroll
-        for (int i = 0; i < NLW; ++i)
-            wreg[i] = (k0 + wl_k < K) ? *reinterpret_cast<const uint4 *>(wsrc[i] + k0) : zero4;
-#pragma unroll
-        for (int i = 0; i < NLX; ++i)
-            xreg[i] = (k0 + xk[i] < K) ? *reinterpret_cast<const uint4 *>(xsrc[i] + k0) : zero4;
-    };
-
+    const u32x4 zero4 = {0u, 0u, 0u, 0u};
+    u32x4 wreg[DEPTH][NLW], xreg[DEPTH][NLX];
     const int nchunks = static_cast<int>((K + KC - 1) / KC);
-    fetch(0);
+    const int nfull = static_cast<int>(K / KC);          // chunks entirely inside K
+
+#define OPMX_FETCH(SET, KCI)                                                                           \
+    do {                                                                                               \
+        const int kci_ = (KCI);                                                                        \
+        if (kci_ < nfull) {                                                                            \
+            const char *wk_ = wb + static_cast<int64_t>(kci_) * (KC * 2);                              \
+            const char *xk_ = xb + static_cast<int64_t>(kci_) * (KC * 2);                              \
+            _Pragma("unroll") for (int i = 0; i < NLW; ++i)                                            \
+                wreg[SET][i] = ld16<NT>(wk_ + (wrow[i] + static_cast<uint32_t>(wl_k * 2)));            \
+            _Pragma("unroll") for (int i = 0; i < NLX; ++i)                                            \
+                xreg[SET][i] = ld16<false>(xk_ + (xrow[i] + static_cast<uint32_t>(xk[i] * 2)));        \
+        } else if (kci_ < nchunks) { /* ragged last chunk: lanes past K read the row start, get 0 */   \
+            const int64_t k0_ = static_cast<int64_t>(kci_) * KC;                                       \
+            _Pragma("unroll") for (int i = 0; i < NLW; ++i) {                                          \
+                const bool in_ = k0_ + wl_k < K;                                                       \
+                const u32x4 v_ = ld16<false>(wb + (wrow[i] + (in_ ? static_cast<uint32_t>((k0_ + wl_k) * 2) : 0u))); \
+                wreg[SET][i] = in_ ? v_ : zero4;                                                       \
+            }                                                                                          \
+            _Pragma("unroll") for (int i = 0; i < NLX; ++i) {                                          \
+                const bool in_ = k0_ + xk[i] < K;                                                      \
+                const u32x4 v_ = ld16<false>(xb + (xrow[i] + (in_ ? static_cast<uint32_t>((k0_ + xk[i]) * 2) : 0u))); \
+                xreg[SET][i] = in_ ? v_ : zero4;                                                       \
+            }                                                                                          \
+        }                                                                                              \
+    } while (0)
+
     const int fr = lane & 15, fg = lane >> 4;   // fragment row (W row / X row) and k group
-    for (int kc = 0; kc < nchunks; ++kc) {
-        char *xcur = xbuf + (kc & 1) * XBUF;
-#pragma unroll
-        for (int i = 0; i < NLW; ++i) *reinterpret_cast<uint4 *>(wstrip + wdst[i]) = wreg[i];
-#pragma unroll
-        for (int i = 0; i < NLX; ++i) *reinterpret_cast<uint4 *>(xcur + xdst[i]) = xreg[i];
-        if (kc + 1 < nchunks) fetch(static_cast<int64_t>(kc + 1) * KC);
-        __syncthreads();
-#pragma unroll
-        for (int s = 0; s < KC / 32; ++s) {
-            const int c = s * 4 + fg;
-            const frag a = *reinterpret_cast<const frag *>(wstrip + fr * RS + c * 16);
-#pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                if (m * 16 < mt.rows) {
-                    const frag b = *reinterpret_cast<const frag *>(xcur + (m * 16 + fr) * RS + c * 16);
-                    acc[m] = Mfma<T>::m16(a, b, acc[m]);
-                }
-            }
+
+#define OPMX_STEP(SET, KCI)                                                                            \
+    do {                                                                                               \
+        char *xcur_ = xbuf + ((KCI)&1) * XBUF;                                                         \
+        _Pragma("unroll") for (int i = 0; i < NLW; ++i)                                                \
+            *reinterpret_cast<u32x4 *>(wstrip + wdst[i]) = wreg[SET][i];                               \
+        _Pragma("unroll") for (int i = 0; i < NLX; ++i)                                                \
+            *reinterpret_cast<u32x4 *>(xcur_ + xdst[i]) = xreg[SET][i];                                \
+        OPMX_FETCH(SET, (KCI) + DEPTH);                                                                \
+        __syncthreads();                                                                               \
+        _Pragma("unroll") for (int s = 0; s < KC / 32; ++s) {                                          \
+            const int c_ = s * 4 + fg;                                                                 \
+            const frag a_ = *reinterpret_cast<const frag *>(wstrip + fr * RS + c_ * 16);               \
+            _Pragma("unroll") for (int m = 0; m < MT; ++m) {                                           \
+                const frag b_ = *reinterpret_cast<const frag *>(xcur_ + (m * 16 + fr) * RS + c_ * 16); \
+                acc[m] = Mfma<T>::m16(a_, b_, acc[m]);                                                 \
+            }                                                                                          \
+        }                                                                                              \
+    } while (0)
+
+    OPMX_FETCH(0, 0);
+    if (DEPTH == 2) OPMX_FETCH(DEPTH - 1, 1);
+    if (DEPTH == 1) {
+        for (int kc = 0; kc < nchunks; ++kc) OPMX_STEP(0, kc);
+    } else {
+        int kc = 0;
+        for (; kc + 1 < nchunks; kc += 2) {
+            OPMX_STEP(0, kc);
+            OPMX_STEP(DEPTH - 1, kc + 1);
         }
+        if (kc < nchunks) OPMX_STEP(0, kc);
     }
+#undef OPMX_STEP
+#undef OPMX_FETCH
 
     // acc[m][i]: W row nbase + fg*4 + i, X row m*16 + fr
 #pragma unroll
@@ -135,13 +174,13 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
     }
 }
 
-template <typename T, int MT, int KC>
+template <typename T, int MT, int KC, int DEPTH, bool NT>
 int stream_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
                   int64_t N, void *Y, hipStream_t s)
 {
     constexpr int RS = KC * 2 + 16;
     constexpr int smem = SW * 16 * RS + 2 * 16 * MT * RS;
-    auto kern = gemm_stream_kernel<T, MT, KC>;
+    auto kern = gemm_stream_kernel<T, MT, KC, DEPTH, NT>;
     static bool attr_done = false;
     if (!attr_done) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -156,19 +195,27 @@ int stream_launch(const void *X, const int64_t *off, const void *W, const void *
     return OPMX_OK;
 }
 
+template <typename T, int KC, int DEPTH, bool NT>
+int stream_pick_mt(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
+                   int64_t N, int64_t m, void *Y, hipStream_t s)
+{
+    if (m <= 16) return stream_launch<T, 1, KC, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
+    if (m <= 32) return stream_launch<T, 2, KC, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
+    return stream_launch<T, 4, 256, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
+}
+
 template <typename T>
 int stream_impl(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
                 int64_t N, int64_t rows_hint, int variant, void *Y, hipStream_t s)
 {
     const int64_t m = rows_hint > 0 ? rows_hint : R;
-    if (variant == 1) {   // 512-wide K chunks
-        if (m <= 16) return stream_launch<T, 1, 512>(X, off, W, B, E, R, K, N, Y, s);
-        if (m <= 32) return stream_launch<T, 2, 512>(X, off, W, B, E, R, K, N, Y, s);
-        return stream_launch<T, 4, 256>(X, off, W, B, E, R, K, N, Y, s);
+    switch (variant) {   // tuning knob; every variant computes the same thing
+        case 1: return stream_pick_mt<T, 256, 1, false>(X, off, W, B, E, R, K, N, m, Y, s);
+        case 2: return stream_pick_mt<T, 512, 1, false>(X, off, W, B, E, R, K, N, m, Y, s);
+        case 3: return stream_pick_mt<T, 256, 2, false>(X, off, W, B, E, R, K, N, m, Y, s);
+        case 4: return stream_pick_mt<T, 512, 2, true>(X, off, W, B, E, R, K, N, m, Y, s);
+        default: return stream_pick_mt<T, 256, 2, true>(X, off, W, B, E, R, K, N, m, Y, s);
     }
-    if (m <= 16) return stream_launch<T, 1, 256>(X, off, W, B, E, R, K, N, Y, s);
-    if (m <= 32) return stream_launch<T, 2, 256>(X, off, W, B, E, R, K, N, Y, s);
-    return stream_launch<T, 4, 256>(X, off, W, B, E, R, K, N, Y, s);
 }
 
 }  // namespace

@@ -86,16 +86,16 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    uint4 ra[LA], rb[LB];
+    u32x4 ra[LA], rb[LB];
     const int nk = static_cast<int>(K / BK);
 #pragma unroll
-    for (int i = 0; i < LA; ++i) ra[i] = *reinterpret_cast<const uint4 *>(Xt + a_src[i]);
+    for (int i = 0; i < LA; ++i) ra[i] = *reinterpret_cast<const u32x4 *>(Xt + a_src[i]);
 #pragma unroll
-    for (int i = 0; i < LB; ++i) rb[i] = *reinterpret_cast<const uint4 *>(We + b_src[i]);
+    for (int i = 0; i < LB; ++i) rb[i] = *reinterpret_cast<const u32x4 *>(We + b_src[i]);
 #pragma unroll
-    for (int i = 0; i < LA; ++i) *reinterpret_cast<uint4 *>(smem + a_dst[i]) = ra[i];
+    for (int i = 0; i < LA; ++i) *reinterpret_cast<u32x4 *>(smem + a_dst[i]) = ra[i];
 #pragma unroll
-    for (int i = 0; i < LB; ++i) *reinterpret_cast<uint4 *>(smem + b_dst[i]) = rb[i];
+    for (int i = 0; i < LB; ++i) *reinterpret_cast<u32x4 *>(smem + b_dst[i]) = rb[i];
     __syncthreads();
 
     const int lrow = lane & 31, lk = lane >> 5;
@@ -106,9 +106,9 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
         if (more) {
             const int64_t ko = static_cast<int64_t>(kt + 1) * BK;
 #pragma unroll
-            for (int i = 0; i < LA; ++i) ra[i] = *reinterpret_cast<const uint4 *>(Xt + a_src[i] + ko);
+            for (int i = 0; i < LA; ++i) ra[i] = *reinterpret_cast<const u32x4 *>(Xt + a_src[i] + ko);
 #pragma unroll
-            for (int i = 0; i < LB; ++i) rb[i] = *reinterpret_cast<const uint4 *>(We + b_src[i] + ko);
+            for (int i = 0; i < LB; ++i) rb[i] = *reinterpret_cast<const u32x4 *>(We + b_src[i] + ko);
         }
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks) {
@@ -127,9 +127,9 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
         }
         if (more) {
 #pragma unroll
-            for (int i = 0; i < LA; ++i) *reinterpret_cast<uint4 *>(nxt + a_dst[i]) = ra[i];
+            for (int i = 0; i < LA; ++i) *reinterpret_cast<u32x4 *>(nxt + a_dst[i]) = ra[i];
 #pragma unroll
-            for (int i = 0; i < LB; ++i) *reinterpret_cast<uint4 *>(nxt + b_dst[i]) = rb[i];
+            for (int i = 0; i < LB; ++i) *reinterpret_cast<u32x4 *>(nxt + b_dst[i]) = rb[i];
         }
         __syncthreads();
     }
