@@ -6,8 +6,9 @@
 // v_mfma_f32_32x32x16_{f16,bf16} are 16-byte loads.  A block owns a BM x BN
 // output tile of ONE expert (tiles never straddle experts; the tile list is
 // derived on the device from expert_offset, no host sync), stages X and W
-// tiles of BK=64 through XOR-swizzled LDS with register prefetch (two LDS
-// buffers, one barrier per k-tile) and accumulates in fp32.  Optional SwiGLU
+// tiles of BK=64 through XOR-swizzled LDS (two LDS buffers, one barrier per
+// k-tile, loads and LDS stores software-pipelined between the MFMA groups) and
+// accumulates in fp32.  Optional SwiGLU
 // epilogue on the accumulators (gate rows i and up rows N/2+i of W are placed
 // in the same lane by the B-tile row order).
 // Semantics: torch_function/MoeColumnParallelLinear.py:61-67,
@@ -21,7 +22,10 @@ constexpr int BK = 64;                 // k elements per LDS tile (128 bytes per
 constexpr int ROWB = BK * 2;           // bytes per LDS row
 constexpr int CH = ROWB / 16;          // 16-byte chunks per row (8)
 
-__device__ __forceinline__ int lds_off(int row, int chunk) { return row * ROWB + ((chunk ^ (row & 7)) << 4); }
+// Byte offset of 16-byte chunk `chunk` of tile row `row`.  Rows are 128 bytes; the
+// XOR with (row>>1)&7 spreads 16 consecutive rows of one chunk column over all
+// sixteen 16-byte bank groups of a 256-byte LDS line pair (conflict-free b128 reads).
+__device__ __forceinline__ int lds_off(int row, int chunk) { return row * ROWB + ((chunk ^ ((row >> 1) & 7)) << 4); }
 
 template <typename T, int BM, int BN, int WM, int WN, bool SWIGLU>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__restrict__ X,
@@ -86,53 +90,77 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    u32x4 ra[LA], rb[LB];
+    // Software pipeline over k-tiles with ONE register set, two LDS buffers and one
+    // barrier per k-tile.  The tile's LA+LB 16-byte quads are spread over the BK/16
+    // MFMA groups of an iteration; in group g of iteration kt the wave
+    //   - reads its fragments of tile kt from LDS buffer kt&1 and issues the MFMAs,
+    //   - stores the quads of slot g (tile kt+1, loaded one iteration ago) into
+    //     LDS buffer (kt+1)&1,
+    //   - reloads the same registers with tile kt+2.
+    // So every global load has a whole iteration to land, and LDS stores and
+    // global loads issue between MFMA groups instead of in a separate phase.
+    constexpr int KS = BK / 16, NQ = LA + LB, QPK = (NQ + KS - 1) / KS;
+    u32x4 rq[NQ];
     const int nk = static_cast<int>(K / BK);
-#pragma unroll
-    for (int i = 0; i < LA; ++i) ra[i] = *reinterpret_cast<const u32x4 *>(Xt + a_src[i]);
-#pragma unroll
-    for (int i = 0; i < LB; ++i) rb[i] = *reinterpret_cast<const u32x4 *>(We + b_src[i]);
-#pragma unroll
-    for (int i = 0; i < LA; ++i) *reinterpret_cast<u32x4 *>(smem + a_dst[i]) = ra[i];
-#pragma unroll
-    for (int i = 0; i < LB; ++i) *reinterpret_cast<u32x4 *>(smem + b_dst[i]) = rb[i];
-    __syncthreads();
-
     const int lrow = lane & 31, lk = lane >> 5;
-    for (int kt = 0; kt < nk; ++kt) {
-        const char *cur = smem + (kt & 1) * STAGE;
-        char *nxt = smem + ((kt + 1) & 1) * STAGE;
-        const bool more = kt + 1 < nk;
-        if (more) {
-            const int64_t ko = static_cast<int64_t>(kt + 1) * BK;
+
+#define OPMX_LOADQ(Q, KT)                                                                          \
+    do {                                                                                           \
+        const int64_t ko_ = static_cast<int64_t>(KT) * BK;                                         \
+        if ((Q) < LA) rq[Q] = *reinterpret_cast<const u32x4 *>(Xt + a_src[(Q) < LA ? (Q) : 0] + ko_); \
+        else rq[Q] = *reinterpret_cast<const u32x4 *>(We + b_src[(Q) < LA ? 0 : (Q)-LA] + ko_);    \
+    } while (0)
+#define OPMX_DRAINQ(Q, BUF)                                                                        \
+    do {                                                                                           \
+        char *dst_ = smem + (BUF)*STAGE;                                                           \
+        if ((Q) < LA) *reinterpret_cast<u32x4 *>(dst_ + a_dst[(Q) < LA ? (Q) : 0]) = rq[Q];        \
+        else *reinterpret_cast<u32x4 *>(dst_ + b_dst[(Q) < LA ? 0 : (Q)-LA]) = rq[Q];              \
+    } while (0)
+#define OPMX_ITER(KT, DRAIN, LOAD)                                                                 \
+    do {                                                                                           \
+        const char *cur_ = smem + ((KT)&1) * STAGE;                                                \
+        _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                        \
+            frag fa[TM], fb[TN];                                                                   \
+            const int chunk = ks * 2 + lk;                                                         \
+            _Pragma("unroll") for (int i = 0; i < TM; ++i)                                         \
+                fa[i] = *reinterpret_cast<const frag *>(cur_ + lds_off(wm * WTM + i * 32 + lrow, chunk)); \
+            _Pragma("unroll") for (int j = 0; j < TN; ++j)                                         \
+                fb[j] = *reinterpret_cast<const frag *>(cur_ + BM * ROWB + lds_off(wn * WTN + j * 32 + lrow, chunk)); \
+            _Pragma("unroll") for (int i = 0; i < TM; ++i)                                         \
+                _Pragma("unroll") for (int j = 0; j < TN; ++j)                                     \
+                    acc[i][j] = Mfma<T>::m32(fa[i], fb[j], acc[i][j]);                             \
+            _Pragma("unroll") for (int qq = 0; qq < QPK; ++qq) {                                   \
+                const int q = ks * QPK + qq;                                                       \
+                if (q < NQ) {                                                                      \
+                    if (DRAIN) OPMX_DRAINQ(q, ((KT) + 1) & 1);                                     \
+                    if (LOAD) OPMX_LOADQ(q, (KT) + 2);                                             \
+                }                                                                                  \
+            }                                                                                      \
+        }                                                                                          \
+        __syncthreads();                                                                           \
+    } while (0)
+
 #pragma unroll
-            for (int i = 0; i < LA; ++i) ra[i] = *reinterpret_cast<const u32x4 *>(Xt + a_src[i] + ko);
+    for (int q = 0; q < NQ; ++q) OPMX_LOADQ(q, 0);
 #pragma unroll
-            for (int i = 0; i < LB; ++i) rb[i] = *reinterpret_cast<const u32x4 *>(We + b_src[i] + ko);
-        }
+    for (int q = 0; q < NQ; ++q) OPMX_DRAINQ(q, 0);
+    if (nk > 1) {
 #pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            frag fa[TM], fb[TN];
-            const int chunk = ks * 2 + lk;
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-                fa[i] = *reinterpret_cast<const frag *>(cur + lds_off(wm * WTM + i * 32 + lrow, chunk));
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                fb[j] = *reinterpret_cast<const frag *>(cur + BM * ROWB + lds_off(wn * WTN + j * 32 + lrow, chunk));
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<T>::m32(fa[i], fb[j], acc[i][j]);
-        }
-        if (more) {
-#pragma unroll
-            for (int i = 0; i < LA; ++i) *reinterpret_cast<u32x4 *>(nxt + a_dst[i]) = ra[i];
-#pragma unroll
-            for (int i = 0; i < LB; ++i) *reinterpret_cast<u32x4 *>(nxt + b_dst[i]) = rb[i];
-        }
-        __syncthreads();
+        for (int q = 0; q < NQ; ++q) OPMX_LOADQ(q, 1);
     }
+    __syncthreads();
+    {
+        int kt = 0;
+        for (; kt + 2 < nk; ++kt) OPMX_ITER(kt, true, true);
+        if (kt + 1 < nk) {
+            OPMX_ITER(kt, true, false);
+            ++kt;
+        }
+        OPMX_ITER(kt, false, false);
+    }
+#undef OPMX_ITER
+#undef OPMX_DRAINQ
+#undef OPMX_LOADQ
 
     // epilogue: acc[i][j][v] is row (v/4)*8 + (lane/32)*4 + v%4, column lane%32 of its 32x32 sub-tile
     const T *be = Bias ? Bias + static_cast<int64_t>(mt.e) * N : nullptr;
@@ -201,6 +229,8 @@ int tiled_impl(const void *X, const int64_t *off, const void *W, const void *B, 
         case 1: return tiled_launch<T, 256, 256, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
         case 2: return tiled_launch<T, 256, 128, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
         case 3: return tiled_launch<T, 256, 256, 2, 4>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        case 4: return tiled_launch<T, 256, 128, 4, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        case 5: return tiled_launch<T, 128, 256, 2, 4>(X, off, W, B, E, R, K, N, epilogue, Y, s);
         default: return tiled_launch<T, 128, 128, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
     }
 }
