@@ -33,6 +33,15 @@ for p in (ROOT, os.path.join(ROOT, "ppl.pmx_amd")):
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, vendor figure
 MFMA_PEAK_TFLOPS = 2500.0      # dense fp16/bf16 MFMA, vendor figure
 
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this program, each scaled by the same counter's reading for a plain copy kernel of known size
+# (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000): profiles/gemm_stream_decode_T32_mixtral8x7b.txt and
+# profiles/gemm_tiled_prefill_T8192_mixtral8x7b.txt.  None where no counter run was made.
+MEASURED_TRAFFIC = {
+    ("decode-T32", False): 1883439104 + 3759718,
+    ("prefill-T8192", False): 2 * 4669289 * 1024 + 921152 * 1024,
+}
+
 SHAPES = {
     "decode": dict(H=4096, E=8, k=2, I=14336, dtype="float16", skew=0.0, name="mixtral-8x7b"),
     "prefill": dict(H=4096, E=8, k=2, I=14336, dtype="float16", skew=4.0, name="mixtral-8x7b"),
@@ -58,6 +67,9 @@ def main():
     ap.add_argument("--fuse-swiglu", action="store_true", help="apply SwiGLU in the gate/up GEMM epilogue")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
+                    help="also run N plain device-to-device copies of the gate/up weight tensor (known size): "
+                         "the reference reading for FETCH_SIZE / WRITE_SIZE counter runs")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (TP=1, no collectives); --gpus {} is not "
@@ -154,6 +166,14 @@ def main():
             for name, a, b in rec:
                 per_op[name] = per_op.get(name, 0.0) + a.elapsed_time(b) * 1e3 / reps
 
+    if args.copy_calibration > 0:
+        dst = torch.empty_like(wu)
+        for _ in range(args.copy_calibration):
+            dst.copy_(wu)
+        torch.cuda.synchronize()
+        print("copy calibration: {} copies of {} bytes (read) + {} bytes (written)".format(
+            args.copy_calibration, wu.numel() * s, wu.numel() * s), file=sys.stderr)
+
     # ---- algorithmic work
     w_bytes_gemm1 = active * 2 * I * H * s
     w_bytes_gemm2 = active * H * I * s
@@ -166,7 +186,8 @@ def main():
     if hbm_bound:
         ach = gemm1_bytes / (gemm1_ms * 1e-3) / 1e9
         roof = dict(bound="hbm", kernel="gate_up_grouped_gemm", achieved=round(ach, 1), peak=HBM_PEAK_GBS,
-                    unit="GB/s", frac=round(ach / HBM_PEAK_GBS, 4), traffic=None,
+                    unit="GB/s", frac=round(ach / HBM_PEAK_GBS, 4),
+                    traffic=MEASURED_TRAFFIC.get((args.workload, args.fuse_swiglu)),
                     algorithmic_bytes=int(gemm1_bytes), launch_ms=round(gemm1_ms, 4))
         lach = layer_bytes / (ms_per_step * 1e-3) / 1e9
         lay = dict(bound="hbm", achieved=round(lach, 1), peak=HBM_PEAK_GBS, unit="GB/s",
@@ -174,7 +195,8 @@ def main():
     else:
         ach = gemm1_flops / (gemm1_ms * 1e-3) / 1e12
         roof = dict(bound="mfma", kernel="gate_up_grouped_gemm", achieved=round(ach, 1), peak=MFMA_PEAK_TFLOPS,
-                    unit="TFLOP/s", frac=round(ach / MFMA_PEAK_TFLOPS, 4), traffic=None,
+                    unit="TFLOP/s", frac=round(ach / MFMA_PEAK_TFLOPS, 4),
+                    traffic=MEASURED_TRAFFIC.get((args.workload, args.fuse_swiglu)),
                     algorithmic_flops=int(gemm1_flops), launch_ms=round(gemm1_ms, 4))
         lach = layer_flops / (ms_per_step * 1e-3) / 1e12
         lay = dict(bound="mfma", achieved=round(lach, 1), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",

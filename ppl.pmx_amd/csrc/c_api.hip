@@ -77,9 +77,13 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
         if (rc != OPMX_OK) return rc;
         return launch_swiglu(ws, R, N / 2, 1.0f, dtype, Y, s);
     }
-    if (choice == 2)
+    if (choice == 2) {
+        // 256x256 tiles (8 waves) once they fill the 256 CUs a few times over, else 128x128.
+        const int64_t big_tiles = (R / 256 + E) * ceil_div(ncols, epilogue == OPMX_EPILOGUE_SWIGLU ? 128 : 256);
+        const int dflt = big_tiles >= 1024 ? 3 : 0;
         return launch_gemm_tiled(X, off, W, B, E, R, K, N, dtype, epilogue,
-                                 env_int("OPMX_MOE_GEMM_TILED_VARIANT", 0), Y, s);
+                                 env_int("OPMX_MOE_GEMM_TILED_VARIANT", dflt), Y, s);
+    }
     return launch_gemm_generic(X, off, W, B, E, R, K, N, dtype, epilogue, Y, s);
 }
 
