@@ -13,6 +13,8 @@
 // in the same lane by the B-tile row order).
 // Semantics: torch_function/MoeColumnParallelLinear.py:61-67,
 // torch_function/MoeRowParallelLinear.py:47-53, torch_function/SwiGLU.py:15-16.
+#include <cstdlib>
+
 #include "moe_gemm.h"
 
 namespace opmx {
@@ -32,7 +34,8 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
                                                                   const int64_t *__restrict__ off,
                                                                   const T *__restrict__ W,
                                                                   const T *__restrict__ Bias, int E, int64_t R,
-                                                                  int64_t K, int64_t N, T *__restrict__ Y)
+                                                                  int64_t K, int64_t N, T *__restrict__ Y,
+                                                                  int ntiles_m, int ntiles_n, int gnx)
 {
     constexpr int NT = WM * WN * 64;
     constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
@@ -48,12 +51,30 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
 
     const int64_t ncols = SWIGLU ? N / 2 : N;
     zero_unowned_rows(Y, R, ncols, off, E);
-    const MTile mt = find_mtile(off, E, R, BM, blockIdx.y, s_off);
+
+    // Block -> tile map.  Workgroups are handed to the 8 XCDs round-robin by linear id and
+    // each XCD has its own L2, so 256 consecutive ids ("a round": 32 per XCD) are laid out
+    // as a gm x (8*gnx) block of tiles in which XCD j owns a compact gm x gnx sub-block:
+    // its 32 resident blocks share gm X-tiles and gnx W-tiles in L2, and all 8 XCDs share
+    // the round's X-tiles through the memory-side cache.  Rounds walk n first, then m.
+    int tile_m, tile_n;
+    if (gnx > 0) {
+        const int gm = 32 / gnx;
+        const int lin = blockIdx.x, xcd = lin & 7, slot = (lin >> 3) & 31, round = lin >> 8;
+        const int rounds_n = (ntiles_n + 8 * gnx - 1) / (8 * gnx);
+        tile_m = (round / rounds_n) * gm + slot % gm;
+        tile_n = (round % rounds_n) * (8 * gnx) + xcd * gnx + slot / gm;
+    } else {                       // plain row-major order, n fastest
+        tile_m = blockIdx.x / ntiles_n;
+        tile_n = blockIdx.x % ntiles_n;
+    }
+    if (tile_m >= ntiles_m || tile_n >= ntiles_n) return;
+    const MTile mt = find_mtile(off, E, R, BM, tile_m, s_off);
     if (mt.rows == 0) return;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
-    const int64_t n0 = static_cast<int64_t>(blockIdx.x) * BNO;
+    const int64_t n0 = static_cast<int64_t>(tile_n) * BNO;
     const T *Xt = X + mt.row0 * K;
     const T *We = W + static_cast<int64_t>(mt.e) * N * K;
 
@@ -90,19 +111,28 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    // Software pipeline over k-tiles with ONE register set, two LDS buffers and one
-    // barrier per k-tile.  The tile's LA+LB 16-byte quads are spread over the BK/16
-    // MFMA groups of an iteration; in group g of iteration kt the wave
-    //   - reads its fragments of tile kt from LDS buffer kt&1 and issues the MFMAs,
-    //   - stores the quads of slot g (tile kt+1, loaded one iteration ago) into
-    //     LDS buffer (kt+1)&1,
-    //   - reloads the same registers with tile kt+2.
-    // So every global load has a whole iteration to land, and LDS stores and
-    // global loads issue between MFMA groups instead of in a separate phase.
-    constexpr int KS = BK / 16, NQ = LA + LB, QPK = (NQ + KS - 1) / KS;
+    // Software pipeline over k-tiles: ONE register set for global->LDS staging, two LDS
+    // buffers, double-buffered MFMA fragments, one barrier per k-tile.
+    // An iteration (tile kt in LDS buffer kt&1) has KS = BK/16 MFMA groups.  Group g
+    //   - prefetches the fragments of group g+1 into the other fragment set,
+    //   - issues its MFMAs on fragments that were fetched one group earlier,
+    //   - (g < KS-1) stores its share of the staging registers (tile kt+1, loaded one
+    //     iteration ago) into LDS buffer (kt+1)&1 and reloads them with tile kt+2.
+    // The barrier sits BEFORE the last group: by then every wave has finished reading
+    // buffer kt&1 (the last group's fragments are already in registers) and writing
+    // buffer (kt+1)&1, so the last group prefetches the first fragments of tile kt+1
+    // while its MFMAs run, and the next iteration may overwrite buffer kt&1.
+    constexpr int KS = BK / 16, NQ = LA + LB, QPK = (NQ + KS - 2) / (KS - 1);
     u32x4 rq[NQ];
+    frag fa[2][TM], fb[2][TN];
     const int nk = static_cast<int>(K / BK);
     const int lrow = lane & 31, lk = lane >> 5;
+    int fa_off[TM], fb_off[TN];      // LDS offsets of this lane's fragments for chunk pair 0
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fa_off[i] = (wm * WTM + i * 32 + lrow) * ROWB;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb_off[j] = BM * ROWB + (wn * WTN + j * 32 + lrow) * ROWB;
+    const int swz = (lrow >> 1) & 7;  // (row>>1)&7 of every fragment row of this lane (rows differ by multiples of 32)
 
 #define OPMX_LOADQ(Q, KT)                                                                          \
     do {                                                                                           \
@@ -116,28 +146,39 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
         if ((Q) < LA) *reinterpret_cast<u32x4 *>(dst_ + a_dst[(Q) < LA ? (Q) : 0]) = rq[Q];        \
         else *reinterpret_cast<u32x4 *>(dst_ + b_dst[(Q) < LA ? 0 : (Q)-LA]) = rq[Q];              \
     } while (0)
-#define OPMX_ITER(KT, DRAIN, LOAD)                                                                 \
+#define OPMX_FRAGS(SET, BUF, G)                                                                    \
     do {                                                                                           \
-        const char *cur_ = smem + ((KT)&1) * STAGE;                                                \
-        _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                        \
-            frag fa[TM], fb[TN];                                                                   \
-            const int chunk = ks * 2 + lk;                                                         \
-            _Pragma("unroll") for (int i = 0; i < TM; ++i)                                         \
-                fa[i] = *reinterpret_cast<const frag *>(cur_ + lds_off(wm * WTM + i * 32 + lrow, chunk)); \
+        const char *src_ = smem + (BUF)*STAGE;                                                     \
+        const int co_ = ((((G)*2 + lk) ^ swz) << 4);                                               \
+        _Pragma("unroll") for (int i = 0; i < TM; ++i)                                             \
+            fa[SET][i] = *reinterpret_cast<const frag *>(src_ + fa_off[i] + co_);                  \
+        _Pragma("unroll") for (int j = 0; j < TN; ++j)                                             \
+            fb[SET][j] = *reinterpret_cast<const frag *>(src_ + fb_off[j] + co_);                  \
+    } while (0)
+#define OPMX_MMA(SET)                                                                              \
+    do {                                                                                           \
+        _Pragma("unroll") for (int i = 0; i < TM; ++i)                                             \
             _Pragma("unroll") for (int j = 0; j < TN; ++j)                                         \
-                fb[j] = *reinterpret_cast<const frag *>(cur_ + BM * ROWB + lds_off(wn * WTN + j * 32 + lrow, chunk)); \
-            _Pragma("unroll") for (int i = 0; i < TM; ++i)                                         \
-                _Pragma("unroll") for (int j = 0; j < TN; ++j)                                     \
-                    acc[i][j] = Mfma<T>::m32(fa[i], fb[j], acc[i][j]);                             \
+                acc[i][j] = Mfma<T>::m32(fa[SET][i], fb[SET][j], acc[i][j]);                       \
+    } while (0)
+#define OPMX_ITER(KT, DRAIN, LOAD, NEXT)                                                           \
+    do {                                                                                           \
+        _Pragma("unroll") for (int g = 0; g < KS - 1; ++g) {                                       \
+            OPMX_FRAGS((g + 1) & 1, (KT)&1, g + 1);                                                \
+            OPMX_MMA(g & 1);                                                                       \
             _Pragma("unroll") for (int qq = 0; qq < QPK; ++qq) {                                   \
-                const int q = ks * QPK + qq;                                                       \
+                const int q = g * QPK + qq;                                                        \
                 if (q < NQ) {                                                                      \
                     if (DRAIN) OPMX_DRAINQ(q, ((KT) + 1) & 1);                                     \
                     if (LOAD) OPMX_LOADQ(q, (KT) + 2);                                             \
                 }                                                                                  \
             }                                                                                      \
+            __builtin_amdgcn_sched_barrier(0);                                                     \
         }                                                                                          \
         __syncthreads();                                                                           \
+        if (NEXT) OPMX_FRAGS(KS & 1, ((KT) + 1) & 1, 0);                                           \
+        OPMX_MMA((KS - 1) & 1);                                                                    \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
     } while (0)
 
 #pragma unroll
@@ -149,16 +190,20 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
         for (int q = 0; q < NQ; ++q) OPMX_LOADQ(q, 1);
     }
     __syncthreads();
+    OPMX_FRAGS(0, 0, 0);
     {
+        static_assert(KS % 2 == 0, "fragment set parity must repeat every k-tile");
         int kt = 0;
-        for (; kt + 2 < nk; ++kt) OPMX_ITER(kt, true, true);
+        for (; kt + 2 < nk; ++kt) OPMX_ITER(kt, true, true, true);
         if (kt + 1 < nk) {
-            OPMX_ITER(kt, true, false);
+            OPMX_ITER(kt, true, false, true);
             ++kt;
         }
-        OPMX_ITER(kt, false, false);
+        OPMX_ITER(kt, false, false, false);
     }
 #undef OPMX_ITER
+#undef OPMX_MMA
+#undef OPMX_FRAGS
 #undef OPMX_DRAINQ
 #undef OPMX_LOADQ
 
@@ -193,7 +238,14 @@ int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B
     constexpr int smem = 2 * (BM + BN) * ROWB;
     const bool sw = epilogue == OPMX_EPILOGUE_SWIGLU;
     const int64_t ncols = sw ? N / 2 : N;
-    dim3 grid(static_cast<unsigned>(ceil_div(ncols, sw ? BN / 2 : BN)), static_cast<unsigned>(max_mtiles(R, E, BM)));
+    const int ntiles_n = static_cast<int>(ceil_div(ncols, sw ? BN / 2 : BN));
+    const int ntiles_m = static_cast<int>(max_mtiles(R, E, BM));
+    int gnx = ntiles_n >= 16 ? 2 : (ntiles_n >= 8 ? 1 : 0);   // n-tiles per XCD per round (measured best)
+    if (const char *v = std::getenv("OPMX_MOE_GEMM_GNX")) gnx = std::atoi(v);   // tuning knob (0: row-major)
+    if (gnx != 0 && gnx != 1 && gnx != 2 && gnx != 4 && gnx != 8 && gnx != 16 && gnx != 32) gnx = 0;
+    const int64_t nblocks = gnx > 0 ? ceil_div(ntiles_n, 8 * gnx) * ceil_div(ntiles_m, 32 / gnx) * 256
+                                    : static_cast<int64_t>(ntiles_n) * ntiles_m;
+    dim3 grid(static_cast<unsigned>(nblocks));
     dim3 block(WM * WN * 64);
     static bool attr_done[2] = {false, false};
     if (sw) {
@@ -205,7 +257,7 @@ int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B
             attr_done[1] = true;
         }
         kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
-                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y));
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_m, ntiles_n, gnx);
     } else {
         auto kern = gemm_tiled_kernel<T, BM, BN, WM, WN, false>;
         if (!attr_done[0]) {
@@ -215,7 +267,7 @@ int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B
             attr_done[0] = true;
         }
         kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
-                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y));
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_m, ntiles_n, gnx);
     }
     OPMX_LAUNCH_CHECK();
     return OPMX_OK;
