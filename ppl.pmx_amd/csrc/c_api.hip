@@ -14,7 +14,9 @@ inline bool dtype_ok(int d) { return d == OPMX_DTYPE_F32 || d == OPMX_DTYPE_F16 
 inline size_t elt(int d) { return d == OPMX_DTYPE_F32 ? 4 : 2; }
 inline hipStream_t st(void *s) { return static_cast<hipStream_t>(s); }
 
-constexpr int64_t kStreamMaxRowsPerExpert = 128;
+// The weight-streaming kernel wins while a row tile of twice the mean rows per expert is
+// at most 64 rows (measured crossover against the 128x128 MFMA tiles on MI355X).
+constexpr int64_t kStreamMaxRowsPerExpert = 64;
 
 int env_int(const char *name, int dflt)
 {
@@ -42,7 +44,7 @@ size_t grouped_gemm_workspace_bytes(int E, int64_t R, int64_t K, int64_t N, int 
     (void)E;
     (void)K;
     // Only the streaming kernel with a fused epilogue stages [R,N] values.
-    if (R <= 0 || N <= 0 || R > kStreamMaxRowsPerExpert * OPMX_MOE_MAX_EXPERTS_PER_TOKEN) return 256;
+    if (R <= 0 || N <= 0 || R > kStreamMaxRowsPerExpert * OPMX_MOE_MAX_EXPERTS) return 256;
     return static_cast<size_t>(ceil_div(R * N * static_cast<int64_t>(elt(dtype)), 256) * 256);
 }
 
@@ -56,7 +58,11 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
     const bool mfma_ok = lowp && K > 0 && K % 8 == 0 && aligned16(X) && aligned16(W) &&
                          N * K < (int64_t{1} << 31) && R * K < (int64_t{1} << 40);
     const bool tiled_ok = mfma_ok && K % 64 == 0;
+    // Row-tile sizing: twice the mean rows per expert, never above what the caller can
+    // guarantee.  An expert with more rows than one tile simply takes several tiles.
     int64_t hint = rows_hint > 0 && rows_hint < R ? rows_hint : R;
+    const int64_t twice_mean = 2 * ceil_div(R, E);
+    if (twice_mean < hint) hint = twice_mean;
     const size_t stage = static_cast<size_t>(R * N) * elt(dtype);
     const bool stream_ws = epilogue == OPMX_EPILOGUE_NONE || (ws && ws_bytes >= stage);
     const int force = forced_kernel();
@@ -78,9 +84,8 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
         return launch_swiglu(ws, R, N / 2, 1.0f, dtype, Y, s);
     }
     if (choice == 2) {
-        // 256x256 tiles (8 waves) once they fill the 256 CUs a few times over, else 128x128.
-        const int64_t big_tiles = (R / 256 + E) * ceil_div(ncols, epilogue == OPMX_EPILOGUE_SWIGLU ? 128 : 256);
-        const int dflt = big_tiles >= 1024 ? 3 : 0;
+        // 256x256 tiles (8 waves) from 128 mean rows per expert on, else 128x128 (measured).
+        const int dflt = R / E >= 128 ? 3 : 0;
         return launch_gemm_tiled(X, off, W, B, E, R, K, N, dtype, epilogue,
                                  env_int("OPMX_MOE_GEMM_TILED_VARIANT", dflt), Y, s);
     }

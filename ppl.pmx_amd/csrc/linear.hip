@@ -2,7 +2,7 @@
 // router gate, N = number of experts).  HBM bound on X: every block streams its
 // tokens' rows once with 16-byte loads and keeps W in cache.
 // Semantics: torch_function/Linear.py:32 of OpenPPL/ppl.pmx.
-#include "common.h"
+#include "moe_gemm.h"
 
 namespace opmx {
 namespace {
@@ -104,6 +104,11 @@ int linear_impl(const void *X_, const void *W_, const void *B_, int64_t Ttok, in
 int launch_linear(const void *X, const void *W, const void *B, int64_t T, int64_t K, int64_t N, int dtype,
                   void *Y, hipStream_t s)
 {
+    // Many tokens: the MFMA tile kernel in dense mode (no expert_offset: one segment [0,T))
+    // reads X once with 128x128 tiles instead of one pass per 8 output features.
+    if ((dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16) && T >= 512 && N > 8 && K % 64 == 0 &&
+        aligned16(X) && aligned16(W) && N * K < (int64_t{1} << 31))
+        return launch_gemm_tiled(X, nullptr, W, B, 1, T, K, N, dtype, OPMX_EPILOGUE_NONE, 0, Y, s);
     switch (dtype) {
         case OPMX_DTYPE_F32: return linear_impl<float>(X, W, B, T, K, N, Y, s);
         case OPMX_DTYPE_F16: return linear_impl<f16>(X, W, B, T, K, N, Y, s);

@@ -50,6 +50,14 @@ struct MTile {
 __device__ __forceinline__ MTile find_mtile(const int64_t *__restrict__ off, int E, int64_t R, int BM,
                                             int64_t tile, int64_t *s_off)
 {
+    if (off == nullptr) {               // dense GEMM: one "expert" owns rows [0, R)
+        MTile d;
+        d.e = 0;
+        d.row0 = tile * BM;
+        const int64_t left = R - d.row0;
+        d.rows = left <= 0 ? 0 : static_cast<int>(left < BM ? left : BM);
+        return d;
+    }
     for (int i = threadIdx.x; i <= E; i += blockDim.x) {
         int64_t v = off[i];
         s_off[i] = v < 0 ? 0 : (v > R ? R : v);
@@ -89,6 +97,7 @@ template <typename T>
 __device__ __forceinline__ void zero_unowned_rows(T *__restrict__ Y, int64_t R, int64_t ncols,
                                                   const int64_t *__restrict__ off, int E)
 {
+    if (off == nullptr) return;
     int64_t lo = off[0], hi = off[E];
     lo = lo < 0 ? 0 : (lo > R ? R : lo);
     hi = hi < lo ? lo : (hi > R ? R : hi);

@@ -195,13 +195,18 @@ int stream_launch(const void *X, const int64_t *off, const void *W, const void *
     return OPMX_OK;
 }
 
-template <typename T, int KC, int DEPTH, bool NT>
+// Row-tile height MT*16 from the rows-per-expert bound m; K-chunk width per height
+// (narrower chunks for taller tiles keep the LDS footprint, hence occupancy, level).
+// 32-row tiles are the measured sweet spot even for a handful of rows; the 16-row
+// instance only serves single-token calls.
+template <typename T, int KC1, int KC2, int KC4, int KC8, int DEPTH, bool NT>
 int stream_pick_mt(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
                    int64_t N, int64_t m, void *Y, hipStream_t s)
 {
-    if (m <= 16) return stream_launch<T, 1, KC, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
-    if (m <= 32) return stream_launch<T, 2, KC, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
-    return stream_launch<T, 4, 256, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
+    if (m <= 2) return stream_launch<T, 1, KC1, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
+    if (m <= 32) return stream_launch<T, 2, KC2, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
+    if (m <= 64) return stream_launch<T, 4, KC4, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
+    return stream_launch<T, 8, KC8, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
 }
 
 template <typename T>
@@ -210,11 +215,12 @@ int stream_impl(const void *X, const int64_t *off, const void *W, const void *B,
 {
     const int64_t m = rows_hint > 0 ? rows_hint : R;
     switch (variant) {   // tuning knob; every variant computes the same thing
-        case 1: return stream_pick_mt<T, 256, 1, false>(X, off, W, B, E, R, K, N, m, Y, s);
-        case 2: return stream_pick_mt<T, 512, 1, false>(X, off, W, B, E, R, K, N, m, Y, s);
-        case 3: return stream_pick_mt<T, 256, 2, false>(X, off, W, B, E, R, K, N, m, Y, s);
-        case 4: return stream_pick_mt<T, 512, 2, true>(X, off, W, B, E, R, K, N, m, Y, s);
-        default: return stream_pick_mt<T, 256, 2, true>(X, off, W, B, E, R, K, N, m, Y, s);
+        case 1: return stream_pick_mt<T, 256, 256, 128, 128, 1, false>(X, off, W, B, E, R, K, N, m, Y, s);
+        case 2: return stream_pick_mt<T, 512, 512, 256, 128, 1, true>(X, off, W, B, E, R, K, N, m, Y, s);
+        case 3: return stream_pick_mt<T, 256, 256, 128, 64, 2, false>(X, off, W, B, E, R, K, N, m, Y, s);
+        case 4: return stream_pick_mt<T, 256, 128, 64, 64, 2, true>(X, off, W, B, E, R, K, N, m, Y, s);
+        case 5: return stream_pick_mt<T, 256, 256, 128, 128, 2, true>(X, off, W, B, E, R, K, N, m, Y, s);
+        default: return stream_pick_mt<T, 256, 256, 128, 64, 2, true>(X, off, W, B, E, R, K, N, m, Y, s);
     }
 }
 

@@ -240,7 +240,8 @@ int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B
     const int64_t ncols = sw ? N / 2 : N;
     const int ntiles_n = static_cast<int>(ceil_div(ncols, sw ? BN / 2 : BN));
     const int ntiles_m = static_cast<int>(max_mtiles(R, E, BM));
-    int gnx = ntiles_n >= 16 ? 2 : (ntiles_n >= 8 ? 1 : 0);   // n-tiles per XCD per round (measured best)
+    // XCD-grouped order only when the n-tiles split evenly over the 8 XCDs (else some XCDs idle)
+    int gnx = ntiles_n % 16 == 0 ? 2 : (ntiles_n % 8 == 0 ? 1 : 0);
     if (const char *v = std::getenv("OPMX_MOE_GEMM_GNX")) gnx = std::atoi(v);   // tuning knob (0: row-major)
     if (gnx != 0 && gnx != 1 && gnx != 2 && gnx != 4 && gnx != 8 && gnx != 16 && gnx != 32) gnx = 0;
     const int64_t nblocks = gnx > 0 ? ceil_div(ntiles_n, 8 * gnx) * ceil_div(ntiles_m, 32 / gnx) * 256

@@ -106,32 +106,36 @@ __device__ __forceinline__ void word_prefix(const uint32_t *bits, int *wordpre, 
     }
 }
 
-// ---- general path, kernel 1: top-k + weights + per-chunk expert histogram ----
+// ---- general path, kernel 1: top-k + weights; one token per lane group ----
 template <typename T>
 __global__ __launch_bounds__(kChunk) void select_topk_kernel(const T *__restrict__ scores, int64_t Ttok,
                                                              int E, int k, int G, int vpl,
                                                              T *__restrict__ weights,
-                                                             int32_t *__restrict__ ids,
-                                                             int32_t *__restrict__ hist)
+                                                             int32_t *__restrict__ ids)
+{
+    const int lig = threadIdx.x % G, grp = threadIdx.x / G, ngrp = kChunk / G;
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * ngrp + grp;
+    if (t >= Ttok) return;                 // whole lane groups leave together
+    int id;
+    float w;
+    route_token(scores + t * E, E, k, G, vpl, lig, id, w);
+    if (lig < k) {
+        ids[t * k + lig] = id;
+        weights[t * k + lig] = from_f32<T>(w);
+    }
+}
+
+// ---- kernel 1b: per-chunk (256 tokens) expert histogram from the picked ids ----
+__global__ __launch_bounds__(kChunk) void select_hist_kernel(const int32_t *__restrict__ ids, int64_t Ttok,
+                                                             int E, int k, int32_t *__restrict__ hist)
 {
     __shared__ uint32_t bits[OPMX_MOE_MAX_EXPERTS * kWords];
-    const int64_t t0 = static_cast<int64_t>(blockIdx.x) * kChunk;
-    const int lig = threadIdx.x % G, grp = threadIdx.x / G, ngrp = kChunk / G;
+    const int tl = threadIdx.x;
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * kChunk + tl;
     zero_bits(bits, E);
     __syncthreads();
-    for (int tl = grp; tl < kChunk; tl += ngrp) {       // uniform trip count inside a wave
-        int64_t t = t0 + tl;
-        if (t < Ttok) {
-            int id;
-            float w;
-            route_token(scores + t * E, E, k, G, vpl, lig, id, w);
-            if (lig < k) {
-                ids[t * k + lig] = id;
-                weights[t * k + lig] = from_f32<T>(w);
-                atomicOr(&bits[id * kWords + (tl >> 5)], 1u << (tl & 31));
-            }
-        }
-    }
+    if (t < Ttok)
+        for (int s = 0; s < k; ++s) atomicOr(&bits[ids[t * k + s] * kWords + (tl >> 5)], 1u << (tl & 31));
     __syncthreads();
     for (int e = threadIdx.x; e < E; e += blockDim.x) {
         int c = 0;
@@ -318,7 +322,10 @@ int select_impl(const void *X_, const void *scores_, int64_t Ttok, int64_t H, in
     char *wsb = static_cast<char *>(ws);
     int32_t *hist = reinterpret_cast<int32_t *>(wsb);
     int32_t *idbuf = ids ? ids : reinterpret_cast<int32_t *>(wsb + ceil_div(sizeof(int32_t) * nchunks * E, 256) * 256);
-    select_topk_kernel<T><<<nchunks, kChunk, 0, s>>>(scores, Ttok, E, k, G, vpl, w, idbuf, hist);
+    select_topk_kernel<T><<<static_cast<unsigned>(ceil_div(Ttok, kChunk / G)), kChunk, 0, s>>>(scores, Ttok, E, k, G,
+                                                                                               vpl, w, idbuf);
+    OPMX_LAUNCH_CHECK();
+    select_hist_kernel<<<nchunks, kChunk, 0, s>>>(idbuf, Ttok, E, k, hist);
     OPMX_LAUNCH_CHECK();
     select_scan_kernel<<<1, 256, 0, s>>>(hist, nchunks, E, R, off);
     OPMX_LAUNCH_CHECK();

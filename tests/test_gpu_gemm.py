@@ -95,7 +95,7 @@ def test_tiled_kernel_variants(variant, dtype):
     run_case("column", sizes, 64, 1000, dtype, False, env, swiglu=True)   # D=500: ragged epilogue tile
 
 
-@pytest.mark.parametrize("variant", ["0", "1", "2", "3", "4"])
+@pytest.mark.parametrize("variant", ["0", "1", "2", "3", "4", "5"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_stream_kernel_variants(variant, dtype):
     env = {"OPMX_MOE_GEMM": "stream", "OPMX_MOE_GEMM_STREAM_VARIANT": variant}
