@@ -19,62 +19,60 @@ __global__ __launch_bounds__(256) void linear_kernel(const T *__restrict__ X, co
     const int64_t t0 = static_cast<int64_t>(blockIdx.x) * TPB;
     const int lane = lane_id(), wave = threadIdx.x / kWave;
 
-    for (int64_t n0 = 0; n0 < N; n0 += kNT) {
-        float acc[TPB][kNT];
+    const int64_t n0 = static_cast<int64_t>(blockIdx.y) * kNT;   // one tile of kNT outputs per block
+    float acc[TPB][kNT];
 #pragma unroll
-        for (int a = 0; a < TPB; ++a)
+    for (int a = 0; a < TPB; ++a)
 #pragma unroll
-            for (int j = 0; j < kNT; ++j) acc[a][j] = 0.0f;
+        for (int j = 0; j < kNT; ++j) acc[a][j] = 0.0f;
 
-        for (int64_t c = static_cast<int64_t>(threadIdx.x) * n; c < K; c += 256 * n) {
-            float xv[TPB][n];
+    for (int64_t c = static_cast<int64_t>(threadIdx.x) * n; c < K; c += 256 * n) {
+        float xv[TPB][n];
 #pragma unroll
-            for (int a = 0; a < TPB; ++a) {
-                const int64_t t = t0 + a < Ttok ? t0 + a : Ttok - 1;
-                if (VEC) {
-                    Vec16<T> v = load16(X + t * K + c);
+        for (int a = 0; a < TPB; ++a) {
+            const int64_t t = t0 + a < Ttok ? t0 + a : Ttok - 1;
+            if (VEC) {
+                Vec16<T> v = load16(X + t * K + c);
 #pragma unroll
-                    for (int i = 0; i < n; ++i) xv[a][i] = to_f32(v.v[i]);
-                } else {
-                    xv[a][0] = to_f32(X[t * K + c]);
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < kNT; ++j) {
-                const int64_t row = n0 + j < N ? n0 + j : N - 1;
-                float wv[n];
-                if (VEC) {
-                    Vec16<T> v = load16(W + row * K + c);
-#pragma unroll
-                    for (int i = 0; i < n; ++i) wv[i] = to_f32(v.v[i]);
-                } else {
-                    wv[0] = to_f32(W[row * K + c]);
-                }
-#pragma unroll
-                for (int a = 0; a < TPB; ++a)
-#pragma unroll
-                    for (int i = 0; i < n; ++i) acc[a][j] += xv[a][i] * wv[i];
+                for (int i = 0; i < n; ++i) xv[a][i] = to_f32(v.v[i]);
+            } else {
+                xv[a][0] = to_f32(X[t * K + c]);
             }
         }
 #pragma unroll
-        for (int a = 0; a < TPB; ++a)
+        for (int j = 0; j < kNT; ++j) {
+            const int64_t row = n0 + j < N ? n0 + j : N - 1;
+            float wv[n];
+            if (VEC) {
+                Vec16<T> v = load16(W + row * K + c);
 #pragma unroll
-            for (int j = 0; j < kNT; ++j) {
-                float v = wave_sum(acc[a][j]);
-                if (lane == 0) red[wave][a * kNT + j] = v;
+                for (int i = 0; i < n; ++i) wv[i] = to_f32(v.v[i]);
+            } else {
+                wv[0] = to_f32(W[row * K + c]);
             }
-        __syncthreads();
-        if (threadIdx.x < TPB * kNT) {
-            const int a = threadIdx.x / kNT, j = threadIdx.x % kNT;
-            if (t0 + a < Ttok && n0 + j < N) {
-                float v = 0.0f;
 #pragma unroll
-                for (int w = 0; w < 256 / kWave; ++w) v += red[w][threadIdx.x];
-                if (B) v += to_f32(B[n0 + j]);
-                Y[(t0 + a) * N + n0 + j] = from_f32<T>(v);
-            }
+            for (int a = 0; a < TPB; ++a)
+#pragma unroll
+                for (int i = 0; i < n; ++i) acc[a][j] += xv[a][i] * wv[i];
         }
-        __syncthreads();
+    }
+#pragma unroll
+    for (int a = 0; a < TPB; ++a)
+#pragma unroll
+        for (int j = 0; j < kNT; ++j) {
+            float v = wave_sum(acc[a][j]);
+            if (lane == 0) red[wave][a * kNT + j] = v;
+        }
+    __syncthreads();
+    if (threadIdx.x < TPB * kNT) {
+        const int a = threadIdx.x / kNT, j = threadIdx.x % kNT;
+        if (t0 + a < Ttok && n0 + j < N) {
+            float v = 0.0f;
+#pragma unroll
+            for (int w = 0; w < 256 / kWave; ++w) v += red[w][threadIdx.x];
+            if (B) v += to_f32(B[n0 + j]);
+            Y[(t0 + a) * N + n0 + j] = from_f32<T>(v);
+        }
     }
 }
 
@@ -87,11 +85,11 @@ int linear_impl(const void *X_, const void *W_, const void *B_, int64_t Ttok, in
     T *Y = static_cast<T *>(Y_);
     const bool vec = K % Vec16<T>::n == 0 && aligned16(X) && aligned16(W);
     if (Ttok >= 1024) {
-        const unsigned grid = static_cast<unsigned>(ceil_div(Ttok, 4));
+        const dim3 grid(static_cast<unsigned>(ceil_div(Ttok, 4)), static_cast<unsigned>(ceil_div(N, kNT)));
         if (vec) linear_kernel<T, 4, true><<<grid, 256, 0, s>>>(X, W, B, Ttok, K, N, Y);
         else linear_kernel<T, 4, false><<<grid, 256, 0, s>>>(X, W, B, Ttok, K, N, Y);
     } else {
-        const unsigned grid = static_cast<unsigned>(Ttok);
+        const dim3 grid(static_cast<unsigned>(Ttok), static_cast<unsigned>(ceil_div(N, kNT)));
         if (vec) linear_kernel<T, 1, true><<<grid, 256, 0, s>>>(X, W, B, Ttok, K, N, Y);
         else linear_kernel<T, 1, false><<<grid, 256, 0, s>>>(X, W, B, Ttok, K, N, Y);
     }

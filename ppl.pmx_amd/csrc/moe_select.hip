@@ -54,21 +54,70 @@ __device__ __forceinline__ void route_token(const T *srow, int E, int k, int G, 
     }
     my_id = -1;
     float my_v = 0.0f;
-    for (int j = 0; j < k; ++j) {
-        uint64_t best = keys[0];
+    if (G == kWave) {
+        // A whole wave routes the token.  Keys are distinct (the id is part of the key),
+        // so "how many keys beat mine" is the key's position in the descending order:
+        // E scalar broadcasts and compares, no k-round dependency chain.  The key of
+        // rank j then moves to lane j through LDS-free cross-lane reads.
+        int rank[kMaxVpl];
 #pragma unroll
-        for (int v = 1; v < kMaxVpl; ++v) best = keys[v] > best ? keys[v] : best;
-        for (int m = G >> 1; m >= 1; m >>= 1) {
-            uint64_t o = shfl_xor_u64(best, m);
-            best = o > best ? o : best;
+        for (int v = 0; v < kMaxVpl; ++v) rank[v] = 0;
+        if (vpl == 1) {                      // E <= 64: one key per lane
+            for (int sl = 0; sl < E; ++sl) {
+                const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[0]), sl);
+                const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[0] >> 32), sl);
+                rank[0] += ((static_cast<uint64_t>(hi) << 32) | lo) > keys[0] ? 1 : 0;
+            }
+        } else {
+#pragma unroll
+            for (int sv = 0; sv < kMaxVpl; ++sv) {
+                if (sv < vpl) {
+                    for (int sl = 0; sl < kWave; ++sl) {
+                        if (sl + sv * kWave >= E) break;
+                        const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[sv]), sl);
+                        const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[sv] >> 32), sl);
+                        const uint64_t other = (static_cast<uint64_t>(hi) << 32) | lo;
+#pragma unroll
+                        for (int v = 0; v < kMaxVpl; ++v) rank[v] += other > keys[v] ? 1 : 0;
+                    }
+                }
+            }
         }
-        int wid = static_cast<int>(0xFFFFFFFFu - static_cast<uint32_t>(best));
+        // lane j < k fetches the key whose rank is j: every lane publishes (rank -> key) by ballot
 #pragma unroll
-        for (int v = 0; v < kMaxVpl; ++v)
-            if (lig + v * G == wid) keys[v] = 0ull;
-        if (lig == j) {
-            my_id = wid;
-            my_v = key_value(static_cast<uint32_t>(best >> 32));
+        for (int v = 0; v < kMaxVpl; ++v) {
+            if (v < vpl) {
+                for (int j = 0; j < k; ++j) {
+                    const uint64_t hit = __ballot(rank[v] == j && keys[v] != 0ull);
+                    if (hit) {
+                        const int src = __ffsll(static_cast<long long>(hit)) - 1;
+                        const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[v]), src);
+                        const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[v] >> 32), src);
+                        if (lig == j) {
+                            my_id = static_cast<int>(0xFFFFFFFFu - lo);
+                            my_v = key_value(hi);
+                        }
+                    }
+                }
+            }
+        }
+    } else {
+        for (int j = 0; j < k; ++j) {
+            uint64_t best = keys[0];
+#pragma unroll
+            for (int v = 1; v < kMaxVpl; ++v) best = keys[v] > best ? keys[v] : best;
+            for (int m = G >> 1; m >= 1; m >>= 1) {
+                uint64_t o = shfl_xor_u64(best, m);
+                best = o > best ? o : best;
+            }
+            int wid = static_cast<int>(0xFFFFFFFFu - static_cast<uint32_t>(best));
+#pragma unroll
+            for (int v = 0; v < kMaxVpl; ++v)
+                if (lig + v * G == wid) keys[v] = 0ull;
+            if (lig == j) {
+                my_id = wid;
+                my_v = key_value(static_cast<uint32_t>(best >> 32));
+            }
         }
     }
     // softmax over the k picked values (MoeSelect.py:41); pick 0 is the maximum
@@ -236,7 +285,7 @@ __global__ __launch_bounds__(256) void select_expand_kernel(const T *__restrict_
 // ---- small-T path: one launch.  Every block routes all T <= kChunk tokens
 // redundantly in LDS, then block b emits the outputs of token b and copies its row.
 template <typename T>
-__global__ __launch_bounds__(kChunk) void select_small_kernel(const T *__restrict__ X,
+__global__ __launch_bounds__(1024) void select_small_kernel(const T *__restrict__ X,
                                                               const T *__restrict__ scores, int Ttok,
                                                               int64_t H, int E, int k, int G, int vpl,
                                                               T *__restrict__ Xp, T *__restrict__ weights,
@@ -249,12 +298,12 @@ __global__ __launch_bounds__(kChunk) void select_small_kernel(const T *__restric
     __shared__ int count[OPMX_MOE_MAX_EXPERTS + 1];
     __shared__ int my_ids[OPMX_MOE_MAX_EXPERTS_PER_TOKEN];
     __shared__ int64_t my_inv[OPMX_MOE_MAX_EXPERTS_PER_TOKEN];
-    const int lig = threadIdx.x % G, grp = threadIdx.x / G, ngrp = kChunk / G;
+    const int lig = threadIdx.x % G, grp = threadIdx.x / G, ngrp = blockDim.x / G;
     const int me = blockIdx.x;                 // the token this block emits
     zero_bits(bits, E);
     __syncthreads();
-    for (int tl = grp; tl < kChunk; tl += ngrp) {
-        if (tl < Ttok) {
+    for (int tl = grp; tl < Ttok; tl += ngrp) {   // whole lane groups iterate together
+        {
             int id;
             float w;
             route_token(scores + static_cast<int64_t>(tl) * E, E, k, G, vpl, lig, id, w);
@@ -313,7 +362,9 @@ int select_impl(const void *X_, const void *scores_, int64_t Ttok, int64_t H, in
         return OPMX_OK;
     }
     if (Ttok <= kChunk && Ttok * G <= kChunk * 8) {
-        select_small_kernel<T><<<static_cast<unsigned>(Ttok), kChunk, 0, s>>>(
+        // wide lane groups (many experts) route few tokens per wave: use a big block
+        const unsigned threads = G >= 32 ? 1024 : kChunk;
+        select_small_kernel<T><<<static_cast<unsigned>(Ttok), threads, 0, s>>>(
             X, scores, static_cast<int>(Ttok), H, E, k, G, vpl, Xp, w, inv, off, ids, vec);
         OPMX_LAUNCH_CHECK();
         return OPMX_OK;
