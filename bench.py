@@ -12,6 +12,8 @@ already resident in HBM.  Prints ONE JSON line:
                        the launch stream, taken inside the timed steps) vs MI355X peak
   layer                the same accounting for the whole layer
   per_op_us            mean duration of each operator (separate untimed pass)
+  device_ceilings      streaming-read GB/s and MFMA TFLOP/s (random fp16 operands) this
+                       device sustains, from the probe ppl.pmx_amd/lib/opmx_device_ceilings
   cpu_baseline         the CPU oracle (PyTorch CPU restatement of the reference
                        operator sequence) on the host cores, bounded sample
 
@@ -67,6 +69,8 @@ def main():
     ap.add_argument("--fuse-swiglu", action="store_true", help="apply SwiGLU in the gate/up GEMM epilogue")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg")
+    ap.add_argument("--no-device-ceilings", action="store_true",
+                    help="skip the probe of the HBM-read / MFMA rates this device sustains")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
                     help="also run N plain device-to-device copies of the gate/up weight tensor (known size): "
                          "the reference reading for FETCH_SIZE / WRITE_SIZE counter runs")
@@ -78,6 +82,18 @@ def main():
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py needs an MI355X (no GPU visible)")
+
+    # What this device sustains (streaming read, MFMA on random operands): a child process,
+    # run before this process touches the GPU.  Context for the roofline fractions only.
+    ceilings = None
+    probe = os.path.join(ROOT, "ppl.pmx_amd", "lib", "opmx_device_ceilings")
+    if not args.no_device_ceilings and os.path.exists(probe):
+        import subprocess
+        try:
+            ceilings = json.loads(subprocess.run([probe], capture_output=True, text=True, timeout=120,
+                                                 check=True).stdout.strip().splitlines()[-1])
+        except Exception as exc:   # the probe is optional
+            print("device ceiling probe failed: {}".format(exc), file=sys.stderr)
     import torch_function as OPMX
     from model_zoo.mixtral.modeling.dynamic_batching.Model import MoeFeedForward
 
@@ -202,6 +218,13 @@ def main():
         lay = dict(bound="mfma", achieved=round(lach, 1), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
                    frac=round(lach / MFMA_PEAK_TFLOPS, 4), algorithmic_flops=int(layer_flops))
 
+    if ceilings:
+        if hbm_bound:
+            roof["measured_ceiling"] = ceilings["hbm_read_nontemporal_GBs"]
+        else:
+            roof["measured_ceiling"] = ceilings["mfma_f16_lds_fed_TFLOPs"]
+        roof["frac_of_measured_ceiling"] = round(roof["achieved"] / roof["measured_ceiling"], 4)
+
     result = {
         "metric": "MoE-layer tokens/sec at Mixtral-8x7B shape, fp16, 1 GPU; % HBM/MFMA roofline",
         "value": round(T / (ms_per_step * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1,
@@ -213,7 +236,7 @@ def main():
             "path": "drop-in operator sequence" + (" + fused SwiGLU epilogue" if args.fuse_swiglu else ""),
             "active_experts": active, "max_expert_share": round(float(counts.max()) / R, 3)},
         "roofline": roof, "layer": lay, "per_op_us": {n: round(v, 1) for n, v in per_op.items()},
-        "device": torch.cuda.get_device_name(0), "cu_count": torch.cuda.get_device_properties(0).multi_processor_count,
+        "device_ceilings": ceilings, "device": torch.cuda.get_device_name(0), "cu_count": torch.cuda.get_device_properties(0).multi_processor_count,
     }
 
     # ---- CPU baseline: the oracle (PyTorch CPU restatement of the reference operator

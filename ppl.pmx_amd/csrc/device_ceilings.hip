@@ -1,0 +1,151 @@
+// Device-ceiling probe for MI355X: what this GPU sustains for (a) a pure streaming
+// read of a weight-sized buffer and (b) an MFMA loop on random fp16 operands,
+// register-fed and LDS-fed.  These are the practical ceilings the grouped-GEMM
+// kernels are compared with in addition to the vendor peaks (8 TB/s, 2.5 PFLOP/s):
+// the engine clock drops under dense MFMA load with toggling operands, so the vendor
+// MFMA peak is not reachable by any kernel on real data.
+// Prints one JSON object.  Build: see Makefile (target ../lib/opmx_device_ceilings).
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+#define CHECK(x)                                                              \
+    do {                                                                      \
+        hipError_t e_ = (x);                                                  \
+        if (e_ != hipSuccess) {                                               \
+            fprintf(stderr, "%s: %s\n", #x, hipGetErrorString(e_));           \
+            return 1;                                                         \
+        }                                                                     \
+    } while (0)
+
+// ---- (a) streaming read: every block reads one contiguous slab, 16 KiB in flight per wave
+template <bool NT>
+__global__ __launch_bounds__(256) void read_kernel(const u32x4 *__restrict__ src, size_t n16_per_block, unsigned *out)
+{
+    const u32x4 *p = src + static_cast<size_t>(blockIdx.x) * n16_per_block;
+    u32x4 acc = {0, 0, 0, 0};
+    for (size_t i = threadIdx.x; i + 15 * 256 < n16_per_block; i += 256 * 16) {
+        u32x4 v[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) v[u] = NT ? __builtin_nontemporal_load(p + i + u * 256) : p[i + u * 256];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) acc ^= v[u];
+    }
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x12345678u) out[0] = 1;
+}
+
+// ---- (b) MFMA 32x32x16 f16 on random operands; LDS_FED: 6 ds_read_b128 per 8 MFMAs
+// (the fragment traffic of a 128x64 wave tile), else two fixed register fragments
+template <bool LDS_FED>
+__global__ __launch_bounds__(512) void mfma_kernel(const _Float16 *__restrict__ src, float *out, int iters)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int tid = threadIdx.x;
+    for (int i = tid; i < 65536 / 16; i += blockDim.x)
+        reinterpret_cast<u32x4 *>(smem)[i] = reinterpret_cast<const u32x4 *>(src)[i + (blockIdx.x & 7) * 4096];
+    __syncthreads();
+    const half8 ra = *reinterpret_cast<const half8 *>(smem + (tid * 16) % 65536);
+    const half8 rb = *reinterpret_cast<const half8 *>(smem + (tid * 16 + 32768) % 65536);
+    float16v acc[8];
+    for (int j = 0; j < 8; ++j)
+        for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+    const int base = (tid >> 6) * 4096 + (tid & 63) * 16;
+    for (int it = 0; it < iters; ++it) {
+        if (LDS_FED) {
+            half8 fa[4], fb[2];
+            const int o = (base + (it & 15) * 3072) & 65520;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) fa[i] = *reinterpret_cast<const half8 *>(smem + ((o + i * 1024) & 65535));
+#pragma unroll
+            for (int i = 0; i < 2; ++i) fb[i] = *reinterpret_cast<const half8 *>(smem + ((o + 32768 + i * 1024) & 65535));
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i * 2 + j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i * 2 + j], 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ra, rb, acc[j], 0, 0, 0);
+        }
+    }
+    float s = 0;
+    for (int j = 0; j < 8; ++j) s += acc[j][0] + acc[j][7];
+    out[blockIdx.x * blockDim.x + tid] = s;
+}
+
+static float best_ms(hipEvent_t e0, hipEvent_t e1, int reps, void (*launch)(void *), void *ctx)
+{
+    float best = 1e30f;
+    for (int r = 0; r < reps; ++r) {
+        (void)hipEventRecord(e0);
+        launch(ctx);
+        (void)hipEventRecord(e1);
+        (void)hipEventSynchronize(e1);
+        float ms = 0;
+        (void)hipEventElapsedTime(&ms, e0, e1);
+        if (r > 0 && ms < best) best = ms;   // first repetition is warm-up
+    }
+    return best;
+}
+
+struct ReadCtx { const u32x4 *src; size_t n16; unsigned *out; int blocks; bool nt; };
+struct MfmaCtx { const _Float16 *src; float *out; int iters; bool lds; };
+
+int main()
+{
+    hipEvent_t e0, e1;
+    CHECK(hipEventCreate(&e0));
+    CHECK(hipEventCreate(&e1));
+    // (a)
+    const size_t bytes = 1879048192ull;   // one Mixtral-8x7B gate/up weight tensor
+    u32x4 *buf;
+    unsigned *flag;
+    CHECK(hipMalloc(&buf, bytes));
+    CHECK(hipMemset(buf, 1, bytes));
+    CHECK(hipMalloc(&flag, 4));
+    const int blocks = 2048;
+    ReadCtx rc{buf, bytes / 16 / blocks, flag, blocks, false};
+    auto read_launch = [](void *c) {
+        ReadCtx *r = static_cast<ReadCtx *>(c);
+        if (r->nt) read_kernel<true><<<r->blocks, 256>>>(r->src, r->n16, r->out);
+        else read_kernel<false><<<r->blocks, 256>>>(r->src, r->n16, r->out);
+    };
+    const double read_plain = bytes / best_ms(e0, e1, 4, read_launch, &rc) / 1e6;
+    rc.nt = true;
+    const double read_nt = bytes / best_ms(e0, e1, 4, read_launch, &rc) / 1e6;
+    // (b)
+    const size_t n = 1 << 20;
+    std::vector<_Float16> h(n);
+    srand(1);
+    for (size_t i = 0; i < n; ++i) h[i] = static_cast<_Float16>(((rand() % 2001) - 1000) * 0.002f);
+    _Float16 *src;
+    float *out;
+    CHECK(hipMalloc(&src, n * 2));
+    CHECK(hipMemcpy(src, h.data(), n * 2, hipMemcpyHostToDevice));
+    CHECK(hipMalloc(&out, 256 * 512 * 4));
+    CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(mfma_kernel<true>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 65536));
+    CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(mfma_kernel<false>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 65536));
+    MfmaCtx mc{src, out, 8000, false};
+    auto mfma_launch = [](void *c) {
+        MfmaCtx *m = static_cast<MfmaCtx *>(c);
+        if (m->lds) mfma_kernel<true><<<256, 512, 65536>>>(m->src, m->out, m->iters);
+        else mfma_kernel<false><<<256, 512, 65536>>>(m->src, m->out, m->iters);
+    };
+    const double flops = 256.0 * 8 * mc.iters * 8 * 32768.0;
+    const double mfma_reg = flops / best_ms(e0, e1, 5, mfma_launch, &mc) / 1e9;
+    mc.lds = true;
+    const double mfma_lds = flops / best_ms(e0, e1, 5, mfma_launch, &mc) / 1e9;
+    CHECK(hipGetLastError());
+    printf("{\"hbm_read_GBs\": %.0f, \"hbm_read_nontemporal_GBs\": %.0f, "
+           "\"mfma_f16_register_fed_TFLOPs\": %.0f, \"mfma_f16_lds_fed_TFLOPs\": %.0f}\n",
+           read_plain, read_nt, mfma_reg, mfma_lds);
+    return 0;
+}

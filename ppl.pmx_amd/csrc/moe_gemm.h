@@ -114,6 +114,8 @@ int launch_gemm_generic(const void *X, const int64_t *off, const void *W, const 
                         int64_t K, int64_t N, int dtype, int epilogue, void *Y, hipStream_t s);
 int launch_gemm_tiled(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
                       int64_t K, int64_t N, int dtype, int epilogue, int variant, void *Y, hipStream_t s);
+int launch_gemm_tiled_dlds(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
+                           int64_t K, int64_t N, int dtype, int epilogue, void *Y, hipStream_t s);
 int launch_gemm_stream(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
                        int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint, int variant, void *Y,
                        hipStream_t s);
