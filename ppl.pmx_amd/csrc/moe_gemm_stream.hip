@@ -20,8 +20,8 @@
 namespace opmx {
 namespace {
 
-constexpr int SW = 4;            // waves per block
-constexpr int SROWS = 16 * SW;   // W rows per block
+// A block has SW waves (4 normally; 1 when the launch would otherwise leave CUs idle)
+// and owns 16*SW consecutive rows of W[e].
 
 template <bool NT> __device__ __forceinline__ u32x4 ld16(const char *p)
 {
@@ -29,13 +29,14 @@ template <bool NT> __device__ __forceinline__ u32x4 ld16(const char *p)
     return *reinterpret_cast<const u32x4 *>(p);
 }
 
-template <typename T, int MT, int KC, int DEPTH, bool NT>
+template <typename T, int MT, int KC, int DEPTH, bool NT, int SW>
 __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restrict__ X,
                                                                const int64_t *__restrict__ off,
                                                                const T *__restrict__ W,
                                                                const T *__restrict__ Bias, int E, int64_t R,
                                                                int64_t K, int64_t N, T *__restrict__ Y)
 {
+    constexpr int SROWS = 16 * SW;               // W rows per block
     constexpr int RS = KC * 2 + 16;              // LDS row stride in bytes (pad 16: conflict-free strips)
     constexpr int RPL = 512 / KC;                // W rows covered by one wave load (1 KiB)
     constexpr int NLW = 16 / RPL;                // W loads per wave per chunk
@@ -174,13 +175,14 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
     }
 }
 
-template <typename T, int MT, int KC, int DEPTH, bool NT>
-int stream_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
-                  int64_t N, void *Y, hipStream_t s)
+template <typename T, int MT, int KC, int DEPTH, bool NT, int SW>
+int stream_launch_sw(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
+                     int64_t N, void *Y, hipStream_t s)
 {
+    constexpr int SROWS = 16 * SW;
     constexpr int RS = KC * 2 + 16;
     constexpr int smem = SW * 16 * RS + 2 * 16 * MT * RS;
-    auto kern = gemm_stream_kernel<T, MT, KC, DEPTH, NT>;
+    auto kern = gemm_stream_kernel<T, MT, KC, DEPTH, NT, SW>;
     static bool attr_done = false;
     if (!attr_done) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -193,6 +195,16 @@ int stream_launch(const void *X, const int64_t *off, const void *W, const void *
                                      static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y));
     OPMX_LAUNCH_CHECK();
     return OPMX_OK;
+}
+
+template <typename T, int MT, int KC, int DEPTH, bool NT>
+int stream_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
+                  int64_t N, void *Y, hipStream_t s)
+{
+    // at most min(R, E) experts are active: with 64-row blocks that is this many work items
+    const int64_t items = ceil_div(N, 64) * (R < E ? R : E);
+    if (MT <= 2 && items < 512) return stream_launch_sw<T, MT, KC, DEPTH, NT, 1>(X, off, W, B, E, R, K, N, Y, s);
+    return stream_launch_sw<T, MT, KC, DEPTH, NT, 4>(X, off, W, B, E, R, K, N, Y, s);
 }
 
 // Row-tile height MT*16 from the rows-per-expert bound m; K-chunk width per height

@@ -110,6 +110,9 @@ def test_stream_kernel_variants(variant, dtype):
     run_case("column", [8, 9, 7, 11, 0, 16, 5, 8], 264, 128, dtype, True, env)      # K % 8 == 0 only
     run_case("column", [8, 9, 7, 11, 0, 16, 5, 8], 512, 256, dtype, True, env, swiglu=True)
     run_case("column", [4] * 64, 256, 128, dtype, False, env)                       # 64 experts
+    # many weight rows: 4-wave blocks (the small cases above run the 1-wave blocks), ragged last slab
+    run_case("column", [8, 9, 7, 11, 0, 16, 5, 8], 256, 4200, dtype, True, env)
+    run_case("row", [30, 2, 17, 0, 32, 1, 25, 21], 512, 4160, dtype, False, env)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
