@@ -49,7 +49,7 @@ import torch
 __all__ = [
     "linear", "topk_lower_id", "moe_select", "moe_column_parallel_linear",
     "moe_row_parallel_linear", "swiglu", "silu", "moe_reduce", "moe_layer",
-    "moe_layer_dense_fp64", "make_inputs", "zipf_router_bias",
+    "moe_layer_dense_fp64", "make_inputs", "zipf_router_bias", "moe_select_as_written",
 ]
 
 
@@ -122,6 +122,33 @@ def moe_select(X: torch.Tensor, scores: torch.Tensor, num_experts: int,
     return out
 
 
+def moe_select_as_written(X, scores, num_experts, num_experts_per_token, acc=torch.float32):
+    """Same results as :func:`moe_select`, but with the bookkeeping done the way the
+    reference does it: one interpreted loop over the R sorted positions to invert the
+    permutation (``MoeSelect.py:49-52``) and a pointer walk over the sorted expert ids
+    for the offsets (``MoeSelect.py:54-60``).  Only used as the "as-written" CPU
+    baseline of the benchmark and to cross-check the vectorised form."""
+    E, k = int(num_experts), int(num_experts_per_token)
+    lead = X.shape[:-1]
+    Xf = X.reshape(-1, X.shape[-1])
+    vals, idx = topk_lower_id(scores.reshape(-1, E), k)
+    w = torch.softmax(_acc(vals, acc), dim=-1).to(scores.dtype)
+    sorted_ids, perm = torch.sort(idx.reshape(-1), stable=True)
+    Xp = Xf.repeat_interleave(k, dim=0)[perm]
+    R = perm.numel()
+    inv = torch.full((R,), -1, dtype=torch.int64)
+    for i in range(R):                                   # per-element tensor get/set
+        inv[perm[i]] = i
+    off = torch.full((E + 1,), -1, dtype=torch.int64)
+    ptr = 0
+    for e in range(E):
+        while ptr < R and sorted_ids[ptr] < e:
+            ptr += 1
+        off[e] = ptr
+    off[E] = R
+    return Xp.view(*lead, k, Xf.shape[-1]), w.view(*lead, k), inv.view(*lead, k), off
+
+
 # --------------------------------------------------------------------------
 # a3 / a5  grouped expert GEMMs
 # --------------------------------------------------------------------------
@@ -192,7 +219,7 @@ def moe_reduce(Y: torch.Tensor, expert_weights: torch.Tensor, invert_permutation
 # --------------------------------------------------------------------------
 def moe_layer(x, Wg, wu, w2, num_experts, num_experts_per_token, *, router_bias=None,
               bu=None, b2=None, round_between_ops: bool = True, acc=torch.float32,
-              scores=None, return_all: bool = False):
+              scores=None, return_all: bool = False, as_written: bool = False):
     """The six-step layer of ``MoeFeedForward.forward`` (fused gate/up form).
 
     ``round_between_ops=True`` rounds every operator output to the input dtype,
@@ -207,8 +234,12 @@ def moe_layer(x, Wg, wu, w2, num_experts, num_experts_per_token, *, router_bias=
     mid = dt if round_between_ops else acc
     if scores is None:
         scores = linear(x, Wg, router_bias, acc=acc, out_dtype=dt)          # 188
-    xe, w, inv, off, idx = moe_select(x, scores, num_experts, num_experts_per_token,
-                                      acc=acc, return_indices=True)         # 191
+    if as_written:
+        xe, w, inv, off = moe_select_as_written(x, scores, num_experts, num_experts_per_token, acc=acc)
+        idx = None
+    else:
+        xe, w, inv, off, idx = moe_select(x, scores, num_experts, num_experts_per_token,
+                                          acc=acc, return_indices=True)     # 191
     x13 = moe_column_parallel_linear(xe, off, wu, bu, acc=acc, out_dtype=mid)   # 198
     a = swiglu(x13, acc=acc, out_dtype=mid)                                 # 200
     y = moe_row_parallel_linear(a, off, w2, b2, acc=acc, out_dtype=mid)     # 208

@@ -174,3 +174,13 @@ def test_reduce_closed_forms():
     w1[:, 2] = 1.0
     out = O.moe_reduce(Y.half(), w1.half(), perm.view(T, k), k)
     assert torch.equal(out, Y.half().view(-1, N)[perm.view(T, k)[:, 2]])
+
+
+def test_as_written_bookkeeping_equals_vectorised():
+    g = torch.Generator().manual_seed(9)
+    for T, E, k in ((1, 8, 2), (37, 8, 2), (20, 64, 8)):
+        X = torch.randn(T, 5, generator=g)
+        s = (torch.randint(-3, 4, (T, E), generator=g).float() * 0.25)
+        a = O.moe_select(X, s, E, k)
+        b = O.moe_select_as_written(X, s, E, k)
+        assert all(torch.equal(p, q) for p, q in zip(a, b))
