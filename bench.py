@@ -46,7 +46,7 @@ MEASURED_TRAFFIC = {
 
 SHAPES = {
     "decode": dict(H=4096, E=8, k=2, I=14336, dtype="float16", skew=0.0, name="mixtral-8x7b"),
-    "prefill": dict(H=4096, E=8, k=2, I=14336, dtype="float16", skew=4.0, name="mixtral-8x7b"),
+    "prefill": dict(H=4096, E=8, k=2, I=14336, dtype="float16", skew=1.5, name="mixtral-8x7b"),
     "fine": dict(H=2048, E=64, k=8, I=1408, dtype="bfloat16", skew=0.0, name="fine-grained-64x8"),
     "8x22b": dict(H=6144, E=8, k=2, I=16384, dtype="float16", skew=0.0, name="mixtral-8x22b-shape"),
 }

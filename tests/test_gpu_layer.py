@@ -101,7 +101,7 @@ def test_mixtral_8x7b_decode(mixtral_8x7b, T):
 def test_mixtral_8x7b_prefill_skewed(mixtral_8x7b, T, full):
     (x, Wg, wu, w2), host = mixtral_8x7b
     E, k = 8, 2
-    bias = O.zipf_router_bias(E, 4.0).half()
+    bias = O.zipf_router_bias(E, 1.5).half()   # shares ~0.43/0.26/0.13/..., all experts active
     g = run_ops(x[:T], Wg, wu, w2, E, k, bias=bias.to(dev()))
     counts = (g["off"][1:] - g["off"][:-1]).cpu()
     assert float(counts.max()) / (T * k) > 0.40, counts.tolist()
