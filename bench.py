@@ -40,8 +40,8 @@ MFMA_PEAK_TFLOPS = 2500.0      # dense fp16/bf16 MFMA, vendor figure
 # (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000): profiles/gemm_stream_decode_T32_mixtral8x7b.txt and
 # profiles/gemm_tiled_prefill_T8192_mixtral8x7b.txt.  None where no counter run was made.
 MEASURED_TRAFFIC = {
-    ("decode-T32", False): 1883439104 + 3759718,
-    ("prefill-T8192", False): 2 * 4669289 * 1024 + 921152 * 1024,
+    ("decode-T32", False): 1883442790 + 3759718,
+    ("prefill-T8192", False): 2 * 5360842 * 1024 + 927043 * 1024,
 }
 
 SHAPES = {
