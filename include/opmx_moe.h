@@ -98,7 +98,10 @@ int opmx_moe_select(const void *X, const void *scores, int64_t T, int64_t H, int
  *   X [R,K], W [E,N,K], B [E,N] or NULL, Y [R,N] (or [R,N/2] with the SwiGLU epilogue).
  * `rows_per_expert_hint` is the largest segment the caller can guarantee
  * (for MoeSelect output: min(R, T)); 0 = unknown.  It only selects between
- * kernel variants, never correctness. */
+ * kernel variants, never correctness.
+ * `workspace` may be NULL with workspace_bytes 0: every epilogue is applied in
+ * registers today; the arguments and the size query are kept so that a future
+ * kernel (e.g. split-K) does not change the ABI. */
 size_t opmx_moe_grouped_gemm_workspace_bytes(int E, int64_t R, int64_t K, int64_t N, int dtype);
 int opmx_moe_column_parallel_linear(const void *X, const int64_t *expert_offset, const void *W,
                                     const void *B, int E, int64_t R, int64_t K, int64_t N,

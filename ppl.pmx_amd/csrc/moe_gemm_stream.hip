@@ -12,7 +12,9 @@
 //    barrier for W);
 //  * the X chunk is shared by the four waves through double-buffered LDS: one
 //    barrier per K-chunk;
-//  * experts with no rows produce no work, so their weights are never touched.
+//  * experts with no rows produce no work, so their weights are never touched;
+//  * optional SwiGLU epilogue: a wave streams 16 gate rows and the 16 matching up rows
+//    (N/2 apart in W[e]) and combines the two accumulators in registers.
 // Semantics: torch_function/MoeColumnParallelLinear.py:61-67 and
 // torch_function/MoeRowParallelLinear.py:47-53 of OpenPPL/ppl.pmx.
 #include "moe_gemm.h"
@@ -29,21 +31,22 @@ template <bool NT> __device__ __forceinline__ u32x4 ld16(const char *p)
     return *reinterpret_cast<const u32x4 *>(p);
 }
 
-template <typename T, int MT, int KC, int DEPTH, bool NT, int SW>
+template <typename T, int MT, int KC, int DEPTH, bool NT, int SW, bool SG>
 __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restrict__ X,
                                                                const int64_t *__restrict__ off,
                                                                const T *__restrict__ W,
                                                                const T *__restrict__ Bias, int E, int64_t R,
                                                                int64_t K, int64_t N, T *__restrict__ Y)
 {
-    constexpr int SROWS = 16 * SW;               // W rows per block
+    constexpr int NG = SG ? 2 : 1;               // row groups per wave: SwiGLU pairs gate rows with up rows
+    constexpr int SROWS = 16 * SW;               // output columns per block
     constexpr int RS = KC * 2 + 16;              // LDS row stride in bytes (pad 16: conflict-free strips)
     constexpr int RPL = 512 / KC;                // W rows covered by one wave load (1 KiB)
     constexpr int NLW = 16 / RPL;                // W loads per wave per chunk
     constexpr int XM = 16 * MT;                  // X rows per tile
     constexpr int CPR = KC / 8;                  // 16-byte chunks per row per K-chunk
     constexpr int NLX = XM * CPR / (SW * 64);    // X loads per thread per chunk
-    constexpr int WSTRIP = 16 * RS;
+    constexpr int WSTRIP = NG * 16 * RS;
     constexpr int XBUF = XM * RS;
     static_assert(XM * CPR % (SW * 64) == 0, "X chunk must divide over the block");
     static_assert(DEPTH == 1 || DEPTH == 2, "one or two chunks in flight");
@@ -52,7 +55,8 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
     extern __shared__ __attribute__((aligned(16))) char smem[];   // [SW][WSTRIP] | [2][XBUF]
     __shared__ int64_t s_off[OPMX_MOE_MAX_EXPERTS + 1];
 
-    zero_unowned_rows(Y, R, N, off, E);
+    const int64_t ND = SG ? N / 2 : N;           // output columns; with SwiGLU W rows n and ND+n pair up
+    zero_unowned_rows(Y, R, ND, off, E);
     const MTile mt = find_mtile(off, E, R, XM, blockIdx.y, s_off);
     if (mt.rows == 0) return;
 
@@ -67,16 +71,18 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
     const char *xb = reinterpret_cast<const char *>(X + mt.row0 * K);
     const int wl_row = lane / (64 / RPL);               // row inside one wave load
     const int wl_k = (lane % (64 / RPL)) * 8;           // k offset inside the chunk
-    uint32_t wrow[NLW];                                 // byte offset of the row start
-    int wdst[NLW];
+    uint32_t wrow[NG][NLW];                             // byte offset of the row start
+    int wdst[NG][NLW];
 #pragma unroll
-    for (int i = 0; i < NLW; ++i) {
-        const int row = i * RPL + wl_row;
-        int64_t n = nbase + row;
-        n = n < N ? n : N - 1;
-        wrow[i] = static_cast<uint32_t>(n * K * 2);
-        wdst[i] = row * RS + wl_k * 2;
-    }
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+        for (int i = 0; i < NLW; ++i) {
+            const int row = i * RPL + wl_row;
+            int64_t n = nbase + row;
+            n = (n < ND ? n : ND - 1) + g * ND;
+            wrow[g][i] = static_cast<uint32_t>(n * K * 2);
+            wdst[g][i] = (g * 16 + row) * RS + wl_k * 2;
+        }
     uint32_t xrow[NLX];
     int xdst[NLX], xk[NLX];
 #pragma unroll
@@ -88,12 +94,14 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
         xk[i] = c * 8;
     }
 
-    float4_t acc[MT];
+    float4_t acc[NG][MT];
 #pragma unroll
-    for (int m = 0; m < MT; ++m) acc[m] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+        for (int m = 0; m < MT; ++m) acc[g][m] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
-    u32x4 wreg[DEPTH][NLW], xreg[DEPTH][NLX];
+    u32x4 wreg[DEPTH][NG][NLW], xreg[DEPTH][NLX];
     const int nchunks = static_cast<int>((K + KC - 1) / KC);
     const int nfull = static_cast<int>(K / KC);          // chunks entirely inside K
 
@@ -103,17 +111,19 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
         if (kci_ < nfull) {                                                                            \
             const char *wk_ = wb + static_cast<int64_t>(kci_) * (KC * 2);                              \
             const char *xk_ = xb + static_cast<int64_t>(kci_) * (KC * 2);                              \
-            _Pragma("unroll") for (int i = 0; i < NLW; ++i)                                            \
-                wreg[SET][i] = ld16<NT>(wk_ + (wrow[i] + static_cast<uint32_t>(wl_k * 2)));            \
+            _Pragma("unroll") for (int g = 0; g < NG; ++g)                                             \
+                _Pragma("unroll") for (int i = 0; i < NLW; ++i)                                        \
+                    wreg[SET][g][i] = ld16<NT>(wk_ + (wrow[g][i] + static_cast<uint32_t>(wl_k * 2)));  \
             _Pragma("unroll") for (int i = 0; i < NLX; ++i)                                            \
                 xreg[SET][i] = ld16<false>(xk_ + (xrow[i] + static_cast<uint32_t>(xk[i] * 2)));        \
         } else if (kci_ < nchunks) { /* ragged last chunk: lanes past K read the row start, get 0 */   \
             const int64_t k0_ = static_cast<int64_t>(kci_) * KC;                                       \
-            _Pragma("unroll") for (int i = 0; i < NLW; ++i) {                                          \
-                const bool in_ = k0_ + wl_k < K;                                                       \
-                const u32x4 v_ = ld16<false>(wb + (wrow[i] + (in_ ? static_cast<uint32_t>((k0_ + wl_k) * 2) : 0u))); \
-                wreg[SET][i] = in_ ? v_ : zero4;                                                       \
-            }                                                                                          \
+            _Pragma("unroll") for (int g = 0; g < NG; ++g)                                             \
+                _Pragma("unroll") for (int i = 0; i < NLW; ++i) {                                      \
+                    const bool in_ = k0_ + wl_k < K;                                                   \
+                    const u32x4 v_ = ld16<false>(wb + (wrow[g][i] + (in_ ? static_cast<uint32_t>((k0_ + wl_k) * 2) : 0u))); \
+                    wreg[SET][g][i] = in_ ? v_ : zero4;                                                \
+                }                                                                                      \
             _Pragma("unroll") for (int i = 0; i < NLX; ++i) {                                          \
                 const bool in_ = k0_ + xk[i] < K;                                                      \
                 const u32x4 v_ = ld16<false>(xb + (xrow[i] + (in_ ? static_cast<uint32_t>((k0_ + xk[i]) * 2) : 0u))); \
@@ -127,18 +137,22 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
 #define OPMX_STEP(SET, KCI)                                                                            \
     do {                                                                                               \
         char *xcur_ = xbuf + ((KCI)&1) * XBUF;                                                         \
-        _Pragma("unroll") for (int i = 0; i < NLW; ++i)                                                \
-            *reinterpret_cast<u32x4 *>(wstrip + wdst[i]) = wreg[SET][i];                               \
+        _Pragma("unroll") for (int g = 0; g < NG; ++g)                                                 \
+            _Pragma("unroll") for (int i = 0; i < NLW; ++i)                                            \
+                *reinterpret_cast<u32x4 *>(wstrip + wdst[g][i]) = wreg[SET][g][i];                     \
         _Pragma("unroll") for (int i = 0; i < NLX; ++i)                                                \
             *reinterpret_cast<u32x4 *>(xcur_ + xdst[i]) = xreg[SET][i];                                \
         OPMX_FETCH(SET, (KCI) + DEPTH);                                                                \
         __syncthreads();                                                                               \
         _Pragma("unroll") for (int s = 0; s < KC / 32; ++s) {                                          \
             const int c_ = s * 4 + fg;                                                                 \
-            const frag a_ = *reinterpret_cast<const frag *>(wstrip + fr * RS + c_ * 16);               \
+            frag a_[NG];                                                                               \
+            _Pragma("unroll") for (int g = 0; g < NG; ++g)                                             \
+                a_[g] = *reinterpret_cast<const frag *>(wstrip + (g * 16 + fr) * RS + c_ * 16);        \
             _Pragma("unroll") for (int m = 0; m < MT; ++m) {                                           \
                 const frag b_ = *reinterpret_cast<const frag *>(xcur_ + (m * 16 + fr) * RS + c_ * 16); \
-                acc[m] = Mfma<T>::m16(a_, b_, acc[m]);                                                 \
+                _Pragma("unroll") for (int g = 0; g < NG; ++g)                                         \
+                    acc[g][m] = Mfma<T>::m16(a_[g], b_, acc[g][m]);                                    \
             }                                                                                          \
         }                                                                                              \
     } while (0)
@@ -158,31 +172,36 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
 #undef OPMX_STEP
 #undef OPMX_FETCH
 
-    // acc[m][i]: W row nbase + fg*4 + i, X row m*16 + fr
+    // acc[g][m][i]: output column nbase + fg*4 + i (W row g*ND + that), X row m*16 + fr
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         const int row = m * 16 + fr;
         if (row >= mt.rows) continue;
-        T *yrow = Y + (mt.row0 + row) * N;
+        T *yrow = Y + (mt.row0 + row) * ND;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int64_t n = nbase + fg * 4 + i;
-            if (n >= N) continue;
-            float v = acc[m][i];
+            if (n >= ND) continue;
+            float v = acc[0][m][i];
             if (Bias) v += to_f32(Bias[static_cast<int64_t>(mt.e) * N + n]);
+            if (SG) {                          // SwiGLU.py:15-16 on the fp32 accumulators, beta = 1
+                float u = acc[NG - 1][m][i];
+                if (Bias) u += to_f32(Bias[static_cast<int64_t>(mt.e) * N + ND + n]);
+                v = u * v * sigmoidf_(v);
+            }
             yrow[n] = from_f32<T>(v);
         }
     }
 }
 
-template <typename T, int MT, int KC, int DEPTH, bool NT, int SW>
+template <typename T, int MT, int KC, int DEPTH, bool NT, int SW, bool SG>
 int stream_launch_sw(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
                      int64_t N, void *Y, hipStream_t s)
 {
     constexpr int SROWS = 16 * SW;
     constexpr int RS = KC * 2 + 16;
-    constexpr int smem = SW * 16 * RS + 2 * 16 * MT * RS;
-    auto kern = gemm_stream_kernel<T, MT, KC, DEPTH, NT, SW>;
+    constexpr int smem = SW * (SG ? 2 : 1) * 16 * RS + 2 * 16 * MT * RS;
+    auto kern = gemm_stream_kernel<T, MT, KC, DEPTH, NT, SW, SG>;
     static bool attr_done = false;
     if (!attr_done) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -190,21 +209,22 @@ int stream_launch_sw(const void *X, const int64_t *off, const void *W, const voi
             return OPMX_ERR_LAUNCH;
         attr_done = true;
     }
-    dim3 grid(static_cast<unsigned>(ceil_div(N, SROWS)), static_cast<unsigned>(max_mtiles(R, E, 16 * MT)));
+    dim3 grid(static_cast<unsigned>(ceil_div(SG ? N / 2 : N, SROWS)), static_cast<unsigned>(max_mtiles(R, E, 16 * MT)));
     kern<<<grid, SW * 64, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
                                      static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y));
     OPMX_LAUNCH_CHECK();
     return OPMX_OK;
 }
 
-template <typename T, int MT, int KC, int DEPTH, bool NT>
+template <typename T, int MT, int KC, int DEPTH, bool NT, bool SG = false>
 int stream_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
                   int64_t N, void *Y, hipStream_t s)
 {
-    // at most min(R, E) experts are active: with 64-row blocks that is this many work items
-    const int64_t items = ceil_div(N, 64) * (R < E ? R : E);
-    if (MT <= 2 && items < 512) return stream_launch_sw<T, MT, KC, DEPTH, NT, 1>(X, off, W, B, E, R, K, N, Y, s);
-    return stream_launch_sw<T, MT, KC, DEPTH, NT, 4>(X, off, W, B, E, R, K, N, Y, s);
+    // at most min(R, E) experts are active: with 64-column blocks that is this many work items
+    const int64_t items = ceil_div(SG ? N / 2 : N, 64) * (R < E ? R : E);
+    if (MT <= 2 && items < 512)
+        return stream_launch_sw<T, MT, KC, DEPTH, NT, 1, SG>(X, off, W, B, E, R, K, N, Y, s);
+    return stream_launch_sw<T, MT, KC, DEPTH, NT, 4, SG>(X, off, W, B, E, R, K, N, Y, s);
 }
 
 // Row-tile height MT*16 from the rows-per-expert bound m; K-chunk width per height
@@ -219,6 +239,18 @@ int stream_pick_mt(const void *X, const int64_t *off, const void *W, const void 
     if (m <= 32) return stream_launch<T, 2, KC2, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
     if (m <= 64) return stream_launch<T, 4, KC4, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
     return stream_launch<T, 8, KC8, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
+}
+
+// SwiGLU epilogue: a wave streams twice the rows, so the K chunks are half as wide.
+template <typename T>
+int stream_swiglu_impl(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
+                       int64_t N, int64_t rows_hint, void *Y, hipStream_t s)
+{
+    const int64_t m = rows_hint > 0 ? rows_hint : R;
+    if (m <= 2) return stream_launch<T, 1, 256, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);
+    if (m <= 32) return stream_launch<T, 2, 128, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);
+    if (m <= 64) return stream_launch<T, 4, 64, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);
+    return stream_launch<T, 8, 64, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);
 }
 
 template <typename T>
@@ -238,12 +270,16 @@ int stream_impl(const void *X, const int64_t *off, const void *W, const void *B,
 
 }  // namespace
 
-// Requires: dtype f16/bf16, K % 8 == 0, 16-byte aligned X and W.  Epilogue NONE only.
+// Requires: dtype f16/bf16, K % 8 == 0, 16-byte aligned X and W.
 int launch_gemm_stream(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
                        int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint, int variant, void *Y,
                        hipStream_t s)
 {
-    if (epilogue != OPMX_EPILOGUE_NONE) return OPMX_ERR_UNSUPPORTED;
+    if (epilogue == OPMX_EPILOGUE_SWIGLU) {
+        if (dtype == OPMX_DTYPE_F16) return stream_swiglu_impl<f16>(X, off, W, B, E, R, K, N, rows_hint, Y, s);
+        if (dtype == OPMX_DTYPE_BF16) return stream_swiglu_impl<bf16>(X, off, W, B, E, R, K, N, rows_hint, Y, s);
+        return OPMX_ERR_UNSUPPORTED;
+    }
     switch (dtype) {
         case OPMX_DTYPE_F16: return stream_impl<f16>(X, off, W, B, E, R, K, N, rows_hint, variant, Y, s);
         case OPMX_DTYPE_BF16: return stream_impl<bf16>(X, off, W, B, E, R, K, N, rows_hint, variant, Y, s);

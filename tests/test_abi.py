@@ -73,4 +73,5 @@ def test_workspace_sizes(lib):
     small = lib.opmx_moe_select_workspace_bytes(32, 8, 2)
     big = lib.opmx_moe_select_workspace_bytes(8192, 8, 2)
     assert small % 256 == 0 and big % 256 == 0 and big >= 8192 * 2 * 4 + 32 * 8 * 4 > small
-    assert lib.opmx_moe_grouped_gemm_workspace_bytes(8, 64, 4096, 28672, 1) >= 64 * 28672 * 2
+    g = lib.opmx_moe_grouped_gemm_workspace_bytes(8, 64, 4096, 28672, 1)
+    assert g >= 256 and g % 256 == 0      # epilogues run in registers: a token workspace is enough
