@@ -7,8 +7,10 @@
 // output tile of ONE expert (tiles never straddle experts; the tile list is
 // derived on the device from expert_offset, no host sync), stages X and W
 // tiles of BK=64 through XOR-swizzled LDS (two LDS buffers, one barrier per
-// k-tile, loads and LDS stores software-pipelined between the MFMA groups) and
-// accumulates in fp32.  Optional SwiGLU
+// k-tile, loads and LDS stores software-pipelined between the MFMA groups; with
+// ILV the instruction order inside a group is pinned to MFMA / fragment read /
+// LDS store / global load round-robin so the matrix pipe never waits behind a
+// burst of memory instructions) and accumulates in fp32.  Optional SwiGLU
 // epilogue on the accumulators (gate rows i and up rows N/2+i of W are placed
 // in the same lane by the B-tile row order).
 // Semantics: torch_function/MoeColumnParallelLinear.py:61-67,
@@ -29,7 +31,7 @@ constexpr int CH = ROWB / 16;          // 16-byte chunks per row (8)
 // sixteen 16-byte bank groups of a 256-byte LDS line pair (conflict-free b128 reads).
 __device__ __forceinline__ int lds_off(int row, int chunk) { return row * ROWB + ((chunk ^ ((row >> 1) & 7)) << 4); }
 
-template <typename T, int BM, int BN, int WM, int WN, bool SWIGLU>
+template <typename T, int BM, int BN, int WM, int WN, bool SWIGLU, bool ILV>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__restrict__ X,
                                                                   const int64_t *__restrict__ off,
                                                                   const T *__restrict__ W,
@@ -123,6 +125,8 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
     // buffer (kt+1)&1, so the last group prefetches the first fragments of tile kt+1
     // while its MFMAs run, and the next iteration may overwrite buffer kt&1.
     constexpr int KS = BK / 16, NQ = LA + LB, QPK = (NQ + KS - 2) / (KS - 1);
+    // first MFMA slot that carries an LDS-store/global-load pair: LDS stores stay behind the group's fragment reads
+    constexpr int ILV0 = TM + TN < TM * TN - QPK ? TM + TN : (TM * TN - QPK > 0 ? TM * TN - QPK : 0);
     u32x4 rq[NQ];
     frag fa[2][TM], fb[2][TN];
     const int nk = static_cast<int>(K / BK);
@@ -173,11 +177,27 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
                     if (LOAD) OPMX_LOADQ(q, (KT) + 2);                                             \
                 }                                                                                  \
             }                                                                                      \
+            if (ILV) {                                                                             \
+                _Pragma("unroll") for (int m = 0; m < TM * TN; ++m) {                              \
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                             \
+                    if (m < TM + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);            \
+                    if (m >= ILV0 && m < ILV0 + QPK && g * QPK + (m - ILV0) < NQ) {                \
+                        if (DRAIN) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);              \
+                        if (LOAD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);               \
+                    }                                                                              \
+                }                                                                                  \
+            }                                                                                      \
             __builtin_amdgcn_sched_barrier(0);                                                     \
         }                                                                                          \
         __syncthreads();                                                                           \
         if (NEXT) OPMX_FRAGS(KS & 1, ((KT) + 1) & 1, 0);                                           \
         OPMX_MMA((KS - 1) & 1);                                                                    \
+        if (ILV && (NEXT)) {                                                                       \
+            _Pragma("unroll") for (int m = 0; m < TM * TN; ++m) {                                  \
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                 \
+                if (m < TM + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                \
+            }                                                                                      \
+        }                                                                                          \
         __builtin_amdgcn_sched_barrier(0);                                                         \
     } while (0)
 
@@ -231,7 +251,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
         }
 }
 
-template <typename T, int BM, int BN, int WM, int WN>
+template <typename T, int BM, int BN, int WM, int WN, bool ILV = false>
 int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
                  int64_t N, int epilogue, void *Y, hipStream_t s)
 {
@@ -250,7 +270,7 @@ int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B
     dim3 block(WM * WN * 64);
     static bool attr_done[2] = {false, false};
     if (sw) {
-        auto kern = gemm_tiled_kernel<T, BM, BN, WM, WN, true>;
+        auto kern = gemm_tiled_kernel<T, BM, BN, WM, WN, true, ILV>;
         if (!attr_done[1]) {
             if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                     smem) != hipSuccess)
@@ -260,7 +280,7 @@ int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B
         kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
                                        static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_m, ntiles_n, gnx);
     } else {
-        auto kern = gemm_tiled_kernel<T, BM, BN, WM, WN, false>;
+        auto kern = gemm_tiled_kernel<T, BM, BN, WM, WN, false, ILV>;
         if (!attr_done[0]) {
             if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                     smem) != hipSuccess)
@@ -278,10 +298,11 @@ template <typename T>
 int tiled_impl(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
                int64_t N, int epilogue, int variant, void *Y, hipStream_t s)
 {
+    // The fixed MFMA / LDS / global-load interleave pays on the 256x256 tiles only.
     switch (variant) {
-        case 1: return tiled_launch<T, 256, 256, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        case 1: return tiled_launch<T, 256, 256, 2, 2, true>(X, off, W, B, E, R, K, N, epilogue, Y, s);
         case 2: return tiled_launch<T, 256, 128, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
-        case 3: return tiled_launch<T, 256, 256, 2, 4>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        case 3: return tiled_launch<T, 256, 256, 2, 4, true>(X, off, W, B, E, R, K, N, epilogue, Y, s);
         case 4: return tiled_launch<T, 256, 128, 4, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
         case 5: return tiled_launch<T, 128, 256, 2, 4>(X, off, W, B, E, R, K, N, epilogue, Y, s);
         default: return tiled_launch<T, 128, 128, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
