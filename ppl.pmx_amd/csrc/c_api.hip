@@ -84,6 +84,8 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
         // 256x256 tiles (8 waves) from 128 mean rows per expert on, else 128x128 (measured).
         const int dflt = R / E >= 128 ? 3 : 0;
         const int variant = env_int("OPMX_MOE_GEMM_TILED_VARIANT", dflt);
+        if (variant >= 7)   // 16x16x32 MFMA kernels: 7 = 256x256/8 waves, 8 = 256x256/4 waves, 9 = 128x128
+            return launch_gemm_tiled16(X, off, W, B, E, R, K, N, dtype, epilogue, variant - 7, Y, s);
         if (variant == 6)   // 256x256 tiles fed by direct-to-LDS loads
             return launch_gemm_tiled_dlds(X, off, W, B, E, R, K, N, dtype, epilogue, Y, s);
         return launch_gemm_tiled(X, off, W, B, E, R, K, N, dtype, epilogue, variant, Y, s);

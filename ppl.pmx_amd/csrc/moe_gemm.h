@@ -23,6 +23,16 @@ template <> struct Mfma<f16> {
     {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
     }
+    // Accumulate in place with the accumulator pinned to an accumulation register quad.
+    // For kernels whose accumulators fill that register file completely: the builtin form
+    // leaves destination and addend as separate values, and with no spare quad the register
+    // allocator then shuffles accumulators through vector registers.  Volatile: keeps
+    // source order against memory instructions, which is how those kernels pin their
+    // MFMA / memory interleave.  The compiler inserts no hazard padding around it.
+    static __device__ __forceinline__ void m16_acc(frag a, frag b, float4_t &c)
+    {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
 };
 template <> struct Mfma<bf16> {
     using frag = bf16x8_t;
@@ -33,6 +43,10 @@ template <> struct Mfma<bf16> {
     static __device__ __forceinline__ float4_t m16(frag a, frag b, float4_t c)
     {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ void m16_acc(frag a, frag b, float4_t &c)
+    {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
 };
 
@@ -114,6 +128,8 @@ int launch_gemm_generic(const void *X, const int64_t *off, const void *W, const 
                         int64_t K, int64_t N, int dtype, int epilogue, void *Y, hipStream_t s);
 int launch_gemm_tiled(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
                       int64_t K, int64_t N, int dtype, int epilogue, int variant, void *Y, hipStream_t s);
+int launch_gemm_tiled16(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
+                        int64_t K, int64_t N, int dtype, int epilogue, int variant, void *Y, hipStream_t s);
 int launch_gemm_tiled_dlds(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
                            int64_t K, int64_t N, int dtype, int epilogue, void *Y, hipStream_t s);
 int launch_gemm_stream(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,

@@ -1,0 +1,967 @@
+// Grouped expert GEMM for gfx950, MFMA-bound regime, on v_mfma_f32_16x16x32.
+//
+//   Y[r, :] = X[r, :] W[e]^T (+ B[e])   for off[e] <= r < off[e+1]
+//
+// Same tiling and pipeline as the 32x32x16 kernel (a block owns a BM x BN tile of
+// one expert, BK=64 k-tiles in XOR-swizzled LDS, two LDS buffers, one barrier per
+// k-tile, one register set staging global->LDS) with two differences that matter
+// on this power-limited part:
+//   - the matrix instruction is 16x16x32, which moves a quarter of the accumulator
+//     registers per instruction: measured ~10% more flops at the same board power
+//     than 32x32x16 on random operands;
+//   - W is the A operand and X the B operand, so a lane ends up with four
+//     consecutive output COLUMNS of one row and the epilogue stores 8 bytes per
+//     lane instead of 2.
+// A k-tile is four MFMA groups (K32 step 0/1 x lower/upper half of the wave's X
+// rows); each group prefetches the fragments of the next one.
+// Semantics: torch_function/MoeColumnParallelLinear.py:61-67,
+// torch_function/MoeRowParallelLinear.py:47-53, torch_function/SwiGLU.py:15-16.
+#include <cstdlib>
+
+#include "moe_gemm.h"
+
+namespace opmx {
+namespace {
+
+constexpr int BK = 64;                 // k elements per LDS tile (128 bytes per row)
+constexpr int ROWB = BK * 2;           // bytes per LDS row
+constexpr int CH = ROWB / 16;          // 16-byte chunks per row (8)
+
+// Byte offset of 16-byte chunk `chunk` of tile row `row`: 16 consecutive rows of one chunk
+// column land in sixteen different 16-byte bank groups (conflict-free b128 fragment reads).
+__device__ __forceinline__ int lds_off(int row, int chunk) { return row * ROWB + ((chunk ^ ((row >> 1) & 7)) << 4); }
+
+// Writes a wave's accumulators.  acc[j][i][v] is output row (X row) i*16 + lane%16 and output
+// column j*16 + (lane/16)*4 + v of the WTM x WTN wave tile: four consecutive columns per lane,
+// stored as one 8-byte word.  With SWIGLU sub-tiles j and j + TNS/2 hold gate and up columns.
+template <typename T, int WTM, int WTN, bool SWIGLU>
+__device__ __forceinline__ void tile_epilogue(float4_t (&acc)[WTN / 16][WTM / 16], const T *__restrict__ Bias,
+                                              T *__restrict__ Y, const MTile &mt, int64_t N, int64_t ncols,
+                                              int64_t n0, int wm, int wn, int lane)
+{
+    constexpr int TMS = WTM / 16, TNS = WTN / 16;
+    const int lrow = lane & 15, lk = lane >> 4;
+    const T *be = Bias ? Bias + static_cast<int64_t>(mt.e) * N : nullptr;
+    const bool vec_ok = (ncols % 4 == 0) && (reinterpret_cast<uintptr_t>(Y) % 8 == 0);
+#pragma unroll
+    for (int i = 0; i < TMS; ++i) {
+        const int row = wm * WTM + i * 16 + lrow;
+        if (row >= mt.rows) continue;
+        T *yrow = Y + (mt.row0 + row) * ncols;
+#pragma unroll
+        for (int j = 0; j < (SWIGLU ? TNS / 2 : TNS); ++j) {
+            const int64_t n = (SWIGLU ? n0 + wn * (WTN / 2) : n0 + wn * WTN) + j * 16 + lk * 4;
+            if (n >= ncols) continue;
+            float val[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int64_t nn = n + v < ncols ? n + v : ncols - 1;
+                float g = acc[j][i][v] + (be ? to_f32(be[nn]) : 0.0f);
+                if (SWIGLU) {
+                    const float up = acc[j + TNS / 2][i][v] + (be ? to_f32(be[ncols + nn]) : 0.0f);
+                    g = up * g * sigmoidf_(g);
+                }
+                val[v] = g;
+            }
+            if (vec_ok && n + 3 < ncols) {
+                T out[4];
+#pragma unroll
+                for (int v = 0; v < 4; ++v) out[v] = from_f32<T>(val[v]);
+                *reinterpret_cast<uint2 *>(yrow + n) = *reinterpret_cast<const uint2 *>(out);
+            } else {
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (n + v < ncols) yrow[n + v] = from_f32<T>(val[v]);
+            }
+        }
+    }
+}
+
+template <typename T, int BM, int BN, int WM, int WN, bool SWIGLU>
+__global__ __launch_bounds__(WM *WN * 64) void gemm_tiled16_kernel(const T *__restrict__ X,
+                                                                    const int64_t *__restrict__ off,
+                                                                    const T *__restrict__ W,
+                                                                    const T *__restrict__ Bias, int E, int64_t R,
+                                                                    int64_t K, int64_t N, T *__restrict__ Y,
+                                                                    int ntiles_m, int ntiles_n, int gnx)
+{
+    constexpr int NT = WM * WN * 64;
+    constexpr int WTM = BM / WM, WTN = BN / WN;          // wave tile: WTM X-rows x WTN W-rows
+    constexpr int TMS = WTM / 16, TNS = WTN / 16;        // 16x16 sub-tiles per wave
+    constexpr int HM = TMS / 2;                          // X sub-tiles per MFMA group
+    constexpr int BNO = SWIGLU ? BN / 2 : BN;            // output columns per tile
+    constexpr int LA = BM * CH / NT, LB = BN * CH / NT;  // 16-byte loads per thread per k-tile
+    constexpr int RSTEP = NT / CH;                       // tile rows between a thread's consecutive loads
+    constexpr int STAGE = (BM + BN) * ROWB;
+    static_assert(BM * CH % NT == 0 && BN * CH % NT == 0, "tile/threads mismatch");
+    static_assert(TMS % 2 == 0 && RSTEP % 16 == 0, "wave tile too small");
+    static_assert(!SWIGLU || TNS % 2 == 0, "SwiGLU needs an even number of n sub-tiles per wave");
+    using frag = typename Mfma<T>::frag;
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    __shared__ int64_t s_off[OPMX_MOE_MAX_EXPERTS + 1];
+
+    const int64_t ncols = SWIGLU ? N / 2 : N;
+    zero_unowned_rows(Y, R, ncols, off, E);
+
+    // Block -> tile map: 256 consecutive block ids (32 per XCD, ids go round-robin over the
+    // 8 XCDs) form a gm x (8*gnx) block of tiles in which XCD j owns a compact gm x gnx
+    // sub-block, so its resident blocks share X- and W-tiles in that XCD's L2.
+    int tile_m, tile_n;
+    if (gnx > 0) {
+        const int gm = 32 / gnx;
+        const int lin = blockIdx.x, xcd = lin & 7, slot = (lin >> 3) & 31, round = lin >> 8;
+        const int rounds_n = (ntiles_n + 8 * gnx - 1) / (8 * gnx);
+        tile_m = (round / rounds_n) * gm + slot % gm;
+        tile_n = (round % rounds_n) * (8 * gnx) + xcd * gnx + slot / gm;
+    } else {
+        tile_m = blockIdx.x / ntiles_n;
+        tile_n = blockIdx.x % ntiles_n;
+    }
+    if (tile_m >= ntiles_m || tile_n >= ntiles_n) return;
+    const MTile mt = find_mtile(off, E, R, BM, tile_m, s_off);
+    if (mt.rows == 0) return;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int64_t n0 = static_cast<int64_t>(tile_n) * BNO;
+    const T *Xt = X + mt.row0 * K;
+    const T *We = W + static_cast<int64_t>(mt.e) * N * K;
+
+    // Staging: load q of a thread covers tile row tid/8 + RSTEP*q, 16-byte chunk tid%8.
+    // RSTEP is a multiple of 16, so the swizzle term is the same for all of them and the
+    // LDS destinations differ by compile-time constants.
+    uint32_t a_src[LA], b_src[LB];   // byte offsets from the (uniform) tile base: scalar base + 32-bit lane offset loads
+    const int srow = tid / CH, sc = tid % CH;
+    const int dst0 = lds_off(srow, sc);
+#pragma unroll
+    for (int i = 0; i < LA; ++i) {
+        const int row = srow + RSTEP * i;
+        const int r = row < mt.rows ? row : mt.rows - 1;
+        a_src[i] = static_cast<uint32_t>((r * K + sc * 8) * 2);
+    }
+#pragma unroll
+    for (int i = 0; i < LB; ++i) {
+        const int row = srow + RSTEP * i;
+        int64_t wrow;
+        if (SWIGLU) {      // wave w's rows: WTN/2 gate rows, then the WTN/2 matching up rows
+            const int w = row / WTN, jj = row % WTN, half = jj / (WTN / 2);
+            int64_t ii = n0 + w * (WTN / 2) + jj % (WTN / 2);
+            ii = ii < ncols ? ii : ncols - 1;
+            wrow = half * ncols + ii;
+        } else {
+            wrow = n0 + row < N ? n0 + row : N - 1;
+        }
+        b_src[i] = static_cast<uint32_t>((wrow * K + sc * 8) * 2);
+    }
+
+    float4_t acc[TNS][TMS];
+#pragma unroll
+    for (int j = 0; j < TNS; ++j)
+#pragma unroll
+        for (int i = 0; i < TMS; ++i)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[j][i][v] = 0.0f;
+
+    // Pipeline over k-tiles (tile kt sits in LDS buffer kt&1).  Group g = 2*s + h of a
+    // k-tile multiplies the K32 step s of the W fragments wf[s] with X fragments xf[h]
+    // (half h of the wave's X sub-tiles), after prefetching the fragments of group g+1:
+    //   g+1 odd : xf[1] <- upper X half of the same step
+    //   g+1 even: xf[0] <- lower X half and wf[s^1] <- W fragments of the next step.
+    // Groups 0..2 also store their share of the staging registers (tile kt+1, loaded one
+    // iteration ago) into buffer (kt+1)&1 and reload them with tile kt+2.  The barrier sits
+    // before group 3, whose prefetch already reads tile kt+1.
+    constexpr int KS = 4, NQ = LA + LB, QPK = (NQ + KS - 2) / (KS - 1), NM = HM * TNS;
+    u32x4 rq[NQ];
+    frag xf[2][HM], wf[2][TNS];
+    const int nk = static_cast<int>(K / BK);
+    const int lrow = lane & 15, lk = lane >> 4;
+    const int swz = (lrow >> 1) & 7;                 // fragment rows differ from lrow by multiples of 16
+    const int x_off = (wm * WTM + lrow) * ROWB;
+    const int w_off = BM * ROWB + (wn * WTN + lrow) * ROWB;
+    const int co0 = ((lk ^ swz) << 4), co1 = (((4 + lk) ^ swz) << 4);
+
+#define OPMX_LOADQ(Q, KT)                                                                          \
+    do {                                                                                           \
+        const int64_t ko_ = static_cast<int64_t>(KT) * BK;                                         \
+        if ((Q) < LA)                                                                              \
+            rq[Q] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(Xt + ko_) +    \
+                                                     a_src[(Q) < LA ? (Q) : 0]);                   \
+        else                                                                                       \
+            rq[Q] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(We + ko_) +    \
+                                                     b_src[(Q) < LA ? 0 : (Q)-LA]);                \
+    } while (0)
+#define OPMX_DRAINQ(Q, BUF)                                                                        \
+    do {                                                                                           \
+        char *dst_ = smem + (BUF)*STAGE + dst0;                                                    \
+        if ((Q) < LA) *reinterpret_cast<u32x4 *>(dst_ + (Q)*RSTEP * ROWB) = rq[Q];                 \
+        else *reinterpret_cast<u32x4 *>(dst_ + BM * ROWB + ((Q)-LA) * RSTEP * ROWB) = rq[Q];       \
+    } while (0)
+    // fragments of group G of the tile in buffer BUF
+#define OPMX_FRAGS(BUF, G)                                                                         \
+    do {                                                                                           \
+        const char *src_ = smem + (BUF)*STAGE + (((G) >> 1) ? co1 : co0);                          \
+        if (((G)&1) == 0) {                                                                        \
+            _Pragma("unroll") for (int i = 0; i < HM; ++i)                                         \
+                xf[0][i] = *reinterpret_cast<const frag *>(src_ + x_off + i * 16 * ROWB);          \
+            _Pragma("unroll") for (int j = 0; j < TNS; ++j)                                        \
+                wf[((G) >> 1) & 1][j] = *reinterpret_cast<const frag *>(src_ + w_off + j * 16 * ROWB); \
+        } else {                                                                                   \
+            _Pragma("unroll") for (int i = 0; i < HM; ++i)                                         \
+                xf[1][i] = *reinterpret_cast<const frag *>(src_ + x_off + (HM + i) * 16 * ROWB);   \
+        }                                                                                          \
+    } while (0)
+#define OPMX_MMA(G)                                                                                \
+    do {                                                                                           \
+        _Pragma("unroll") for (int i = 0; i < HM; ++i)                                             \
+            _Pragma("unroll") for (int j = 0; j < TNS; ++j)                                        \
+                acc[j][((G)&1) * HM + i] =                                                         \
+                    Mfma<T>::m16(wf[((G) >> 1) & 1][j], xf[(G)&1][i], acc[j][((G)&1) * HM + i]);   \
+    } while (0)
+    // Pin the order inside a group: one fragment read behind each of the first MFMAs, then
+    // one LDS-store / global-load pair behind each of the following ones.
+#define OPMX_ORDER(NREAD, NPAIR, DRAIN, LOAD)                                                      \
+    do {                                                                                           \
+        _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                     \
+            if (m < (NREAD)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                    \
+            const int p0 = (NREAD) < NM - (NPAIR) ? (NREAD) : (NM - (NPAIR) > 0 ? NM - (NPAIR) : 0); \
+            if (m >= p0 && m < p0 + (NPAIR)) {                                                     \
+                if (DRAIN) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                      \
+                if (LOAD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                       \
+            }                                                                                      \
+        }                                                                                          \
+    } while (0)
+#define OPMX_ITER(KT, DRAIN, LOAD, NEXT)                                                           \
+    do {                                                                                           \
+        _Pragma("unroll") for (int g = 0; g < KS - 1; ++g) {                                       \
+            OPMX_FRAGS((KT)&1, g + 1);                                                             \
+            OPMX_MMA(g);                                                                           \
+            _Pragma("unroll") for (int qq = 0; qq < QPK; ++qq) {                                   \
+                const int q = g * QPK + qq;                                                        \
+                if (q < NQ) {                                                                      \
+                    if (DRAIN) OPMX_DRAINQ(q, ((KT) + 1) & 1);                                     \
+                    if (LOAD) OPMX_LOADQ(q, (KT) + 2);                                             \
+                }                                                                                  \
+            }                                                                                      \
+            OPMX_ORDER(((g + 1) & 1) ? HM : HM + TNS,                                              \
+                       (NQ - g * QPK < QPK ? (NQ - g * QPK > 0 ? NQ - g * QPK : 0) : QPK), DRAIN, LOAD); \
+            __builtin_amdgcn_sched_barrier(0);                                                     \
+        }                                                                                          \
+        __syncthreads();                                                                           \
+        if (NEXT) OPMX_FRAGS(((KT) + 1) & 1, 0);                                                   \
+        OPMX_MMA(KS - 1);                                                                          \
+        if (NEXT) OPMX_ORDER(HM + TNS, 0, false, false);                                           \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+    } while (0)
+
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) OPMX_LOADQ(q, 0);
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) OPMX_DRAINQ(q, 0);
+    if (nk > 1) {
+#pragma unroll
+        for (int q = 0; q < NQ; ++q) OPMX_LOADQ(q, 1);
+    }
+    __syncthreads();
+    OPMX_FRAGS(0, 0);
+    {
+        int kt = 0;
+        for (; kt + 2 < nk; ++kt) OPMX_ITER(kt, true, true, true);
+        if (kt + 1 < nk) {
+            OPMX_ITER(kt, true, false, true);
+            ++kt;
+        }
+        OPMX_ITER(kt, false, false, false);
+    }
+#undef OPMX_ITER
+#undef OPMX_ORDER
+#undef OPMX_MMA
+#undef OPMX_FRAGS
+#undef OPMX_DRAINQ
+#undef OPMX_LOADQ
+
+    tile_epilogue<T, WTM, WTN, SWIGLU>(acc, Bias, Y, mt, N, ncols, n0, wm, wn, lane);
+}
+
+// ---------------------------------------------------------------------------------------
+// Direct-to-LDS variant.  Operand tiles are written into LDS by global_load_lds_dwordx4
+// (1 KiB per wave instruction: lane l lands at base + 16*l), so staging costs no VGPRs and
+// no ds_write.  Same LDS layout as above (rows of BK=64, chunk XOR (row>>1)&7); the XOR is
+// applied by choosing which global chunk a lane fetches: a wave load covers 8 tile rows,
+// lane l fetches chunk (l%8) ^ ((row>>1)&7) of row l/8, i.e. whole 128-byte lines.
+// Two LDS buffers, one barrier per k-tile, placed before the last of the four MFMA groups:
+//   - before it, every wave has read all fragments of buffer kt&1 (those of group 3 are in
+//     registers) and waited for its own loads of tile kt+1 (vmcnt(0));
+//   - after it, group 3 runs while the first fragments of tile kt+1 are read and the first
+//     half of the loads of tile kt+2 is issued into buffer kt&1; the second half follows in
+//     group 0 of the next k-tile, leaving groups 1-2 for the data to land.
+// ASM: the MFMAs are volatile asm with the accumulator tied to an accumulation-register quad
+// and the source order is the issue order (needed when the accumulators fill all 256 of those
+// registers, WM*WN = 4); otherwise compiler builtins plus sched_group_barrier directives.
+#define OPMX_GPTR(p) ((const void __attribute__((address_space(1))) *)(p))
+#define OPMX_LPTR(p) ((void __attribute__((address_space(3))) *)(p))
+
+// Block barrier WITHOUT a memory fence (a fence would wait for every in-flight direct-to-LDS
+// load).  The caller orders explicitly: s_waitcnt vmcnt(0) for the tile it publishes,
+// lgkmcnt(0) here for its own LDS reads of the buffer being retired.
+__device__ __forceinline__ void barrier_no_fence()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+template <typename T, int BM, int BN, int WM, int WN, bool SWIGLU, bool ASM>
+__global__ __launch_bounds__(WM *WN * 64) void gemm_tiled16_dlds_kernel(const T *__restrict__ X,
+                                                                         const int64_t *__restrict__ off,
+                                                                         const T *__restrict__ W,
+                                                                         const T *__restrict__ Bias, int E,
+                                                                         int64_t R, int64_t K, int64_t N,
+                                                                         T *__restrict__ Y, int ntiles_m,
+                                                                         int ntiles_n, int gnx)
+{
+    constexpr int NW = WM * WN;
+    constexpr int WTM = BM / WM, WTN = BN / WN, TMS = WTM / 16, TNS = WTN / 16, HM = TMS / 2;
+    constexpr int BNO = SWIGLU ? BN / 2 : BN;
+    constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW;   // 1 KiB wave loads per wave per k-tile
+    constexpr int NL = LA + LB, NLH = NL / 2, NM = HM * TNS;
+    constexpr int STAGE = (BM + BN) * ROWB;
+    static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0 && NL % 2 == 0, "tile/waves mismatch");
+    static_assert(HM + TNS + NLH <= NM, "not enough MFMA slots in a group for its memory instructions");
+    static_assert(!SWIGLU || TNS % 2 == 0, "SwiGLU needs an even number of n sub-tiles per wave");
+    using frag = typename Mfma<T>::frag;
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    __shared__ int64_t s_off[OPMX_MOE_MAX_EXPERTS + 1];
+
+    const int64_t ncols = SWIGLU ? N / 2 : N;
+    zero_unowned_rows(Y, R, ncols, off, E);
+    int tile_m, tile_n;
+    if (gnx > 0) {
+        const int gm = 32 / gnx;
+        const int lin = blockIdx.x, xcd = lin & 7, slot = (lin >> 3) & 31, round = lin >> 8;
+        const int rounds_n = (ntiles_n + 8 * gnx - 1) / (8 * gnx);
+        tile_m = (round / rounds_n) * gm + slot % gm;
+        tile_n = (round % rounds_n) * (8 * gnx) + xcd * gnx + slot / gm;
+    } else {
+        tile_m = blockIdx.x / ntiles_n;
+        tile_n = blockIdx.x % ntiles_n;
+    }
+    if (tile_m >= ntiles_m || tile_n >= ntiles_n) return;
+    const MTile mt = find_mtile(off, E, R, BM, tile_m, s_off);
+    if (mt.rows == 0) return;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int64_t n0 = static_cast<int64_t>(tile_n) * BNO;
+    const char *xb = reinterpret_cast<const char *>(X + mt.row0 * K);
+    const char *wb = reinterpret_cast<const char *>(W + static_cast<int64_t>(mt.e) * N * K);
+
+    // this lane's share of the wave loads: tile row 8*(wave*L+i) + lane/8, LDS slot lane%8
+    const int lrow8 = lane >> 3, slot = lane & 7;
+    uint32_t a_src[LA], b_src[LB];     // byte offsets from xb / wb at k = 0
+#pragma unroll
+    for (int i = 0; i < LA; ++i) {
+        const int row = (wave * LA + i) * 8 + lrow8;
+        const int r = row < mt.rows ? row : mt.rows - 1;
+        const int c = slot ^ ((row >> 1) & 7);
+        a_src[i] = static_cast<uint32_t>((r * K + c * 8) * 2);
+    }
+#pragma unroll
+    for (int i = 0; i < LB; ++i) {
+        const int row = (wave * LB + i) * 8 + lrow8;
+        int64_t wrow;
+        if (SWIGLU) {
+            const int w = row / WTN, jj = row % WTN, half = jj / (WTN / 2);
+            int64_t ii = n0 + w * (WTN / 2) + jj % (WTN / 2);
+            ii = ii < ncols ? ii : ncols - 1;
+            wrow = half * ncols + ii;
+        } else {
+            wrow = n0 + row < N ? n0 + row : N - 1;
+        }
+        const int c = slot ^ ((row >> 1) & 7);
+        b_src[i] = static_cast<uint32_t>((wrow * K + c * 8) * 2);
+    }
+    const int a_lds = wave * LA * 1024, b_lds = BM * ROWB + wave * LB * 1024;   // wave-uniform
+
+    float4_t acc[TNS][TMS];
+#pragma unroll
+    for (int j = 0; j < TNS; ++j)
+#pragma unroll
+        for (int i = 0; i < TMS; ++i)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[j][i][v] = 0.0f;
+
+    const int nk = static_cast<int>(K / BK);
+    const int lrow = lane & 15, lk = lane >> 4;
+    const int swz = (lrow >> 1) & 7;
+    const int x_off = (wm * WTM + lrow) * ROWB;
+    const int w_off = BM * ROWB + (wn * WTN + lrow) * ROWB;
+    const int co0 = ((lk ^ swz) << 4), co1 = (((4 + lk) ^ swz) << 4);
+    frag xf[2][HM], wf[2][TNS];
+
+    // wave load Q of tile KT into buffer BUF: Q < LA -> X rows, else W rows
+#define OPMX_ISSUE1(KT, BUF, Q)                                                                    \
+    do {                                                                                           \
+        char *st_ = smem + (BUF)*STAGE;                                                            \
+        const int64_t kb_ = static_cast<int64_t>(KT) * ROWB;                                       \
+        if ((Q) < LA)                                                                              \
+            __builtin_amdgcn_global_load_lds(OPMX_GPTR(xb + kb_ + a_src[(Q) < LA ? (Q) : 0]),      \
+                                             OPMX_LPTR(st_ + a_lds + (Q)*1024), 16, 0, 0);         \
+        else                                                                                       \
+            __builtin_amdgcn_global_load_lds(OPMX_GPTR(wb + kb_ + b_src[(Q) < LA ? 0 : (Q)-LA]),   \
+                                             OPMX_LPTR(st_ + b_lds + ((Q)-LA) * 1024), 16, 0, 0);  \
+    } while (0)
+    // fragment F of MFMA group G (= 2*step + X half) of the tile in buffer BUF.  Even groups
+    // need HM lower-half X fragments and the TNS W fragments of their step, odd groups the HM
+    // upper-half X fragments.
+#define OPMX_FRAG1(BUF, G, F)                                                                      \
+    do {                                                                                           \
+        const char *src_ = smem + (BUF)*STAGE + (((G) >> 1) ? co1 : co0);                          \
+        if (((G)&1) != 0)                                                                          \
+            xf[1][(F) < HM ? (F) : 0] = *reinterpret_cast<const frag *>(src_ + x_off + (HM + (F)) * 16 * ROWB); \
+        else if ((F) < HM)                                                                         \
+            xf[0][(F) < HM ? (F) : 0] = *reinterpret_cast<const frag *>(src_ + x_off + (F)*16 * ROWB); \
+        else                                                                                       \
+            wf[((G) >> 1) & 1][(F) < HM ? 0 : (F)-HM] =                                            \
+                *reinterpret_cast<const frag *>(src_ + w_off + ((F)-HM) * 16 * ROWB);              \
+    } while (0)
+#define OPMX_NFRAG(G) ((((G)&1) != 0) ? HM : HM + TNS)
+    // MFMA group G: MFMA m, then (in this order) one fragment read of group G+1 while there are
+    // any (NREAD, from buffer FBUF), then one wave load (NLOAD of them, numbers LQ0.., tile LKT
+    // into buffer LBUF).
+#define OPMX_GROUP(G, FBUF, NREAD, LKT, LBUF, LQ0, NLOAD)                                          \
+    do {                                                                                           \
+        _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
+            if (ASM)                                                                               \
+                Mfma<T>::m16_acc(wf[((G) >> 1) & 1][m % TNS], xf[(G)&1][m / TNS],                  \
+                                 acc[m % TNS][((G)&1) * HM + m / TNS]);                            \
+            else                                                                                   \
+                acc[m % TNS][((G)&1) * HM + m / TNS] =                                             \
+                    Mfma<T>::m16(wf[((G) >> 1) & 1][m % TNS], xf[(G)&1][m / TNS],                  \
+                                 acc[m % TNS][((G)&1) * HM + m / TNS]);                            \
+            if (m < (NREAD)) OPMX_FRAG1(FBUF, ((G) + 1) & 3, m);                                   \
+            else if (m - (NREAD) < (NLOAD)) OPMX_ISSUE1(LKT, LBUF, (LQ0) + m - (NREAD));           \
+        }                                                                                          \
+        if (!ASM) {                                                                                \
+            _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                       \
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                 \
+                if (m < (NREAD)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                \
+                else if (m - (NREAD) < (NLOAD)) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0); \
+            }                                                                                      \
+        }                                                                                          \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+    } while (0)
+    // k-tile KT in buffer KT&1.  LD1: tile kt+1 exists (its second-half loads go out in group
+    // 0, its first fragments are read in group 3).  LD2: tile kt+2 exists.
+#define OPMX_ITER(KT, LD1, LD2)                                                                    \
+    do {                                                                                           \
+        OPMX_GROUP(0, (KT)&1, OPMX_NFRAG(1), (KT) + 1, ((KT) + 1) & 1, NLH, (LD1) ? NL - NLH : 0); \
+        OPMX_GROUP(1, (KT)&1, OPMX_NFRAG(2), 0, 0, 0, 0);                                          \
+        OPMX_GROUP(2, (KT)&1, OPMX_NFRAG(3), 0, 0, 0, 0);                                          \
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                           \
+        barrier_no_fence();                                                                        \
+        OPMX_GROUP(3, ((KT) + 1) & 1, (LD1) ? OPMX_NFRAG(0) : 0, (KT) + 2, (KT)&1, 0, (LD2) ? NLH : 0); \
+    } while (0)
+
+    // prologue: tile 0 -> buffer 0; first half of tile 1 -> buffer 1; fragments of group 0
+#pragma unroll
+    for (int q = 0; q < NL; ++q) OPMX_ISSUE1(0, 0, q);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    barrier_no_fence();
+    if (nk > 1) {
+#pragma unroll
+        for (int q = 0; q < NLH; ++q) OPMX_ISSUE1(1, 1, q);
+    }
+#pragma unroll
+    for (int f = 0; f < HM + TNS; ++f) OPMX_FRAG1(0, 0, f);
+    {
+        int kt = 0;
+        for (; kt + 2 < nk; ++kt) OPMX_ITER(kt, true, true);
+        if (kt + 1 < nk) {
+            OPMX_ITER(kt, true, false);
+            ++kt;
+        }
+        OPMX_ITER(kt, false, false);
+    }
+#undef OPMX_ITER
+#undef OPMX_GROUP
+#undef OPMX_NFRAG
+#undef OPMX_FRAG1
+#undef OPMX_ISSUE1
+
+    // asm MFMAs are opaque to the compiler's hazard padding: let the last ones retire before
+    // the accumulators are read
+    if (ASM) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    tile_epilogue<T, WTM, WTN, SWIGLU>(acc, Bias, Y, mt, N, ncols, n0, wm, wn, lane);
+}
+
+// Raw buffer descriptor over [base, base + 4 GiB): loads through it take a scalar base, a
+// scalar offset and a 32-bit lane offset.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t raw_descriptor(const void *base)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, static_cast<int>(0xFFFFFFFFu), 0x00020000);
+}
+
+// 16 bytes per lane from descriptor + soff + voff straight into LDS at lds + 16*lane (lds is
+// wave-uniform).
+__device__ __forceinline__ void load_to_lds_16(__amdgpu_buffer_rsrc_t r, char *lds, uint32_t voff, int soff)
+{
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, OPMX_LPTR(lds), 16, voff, soff, 0, 0);
+}
+
+// Linear tile id -> (row tile of one expert, column tile), in the XCD-grouped order described
+// at the tile map of the kernels above.  mt.rows == 0 when the id names no work.  s_off is the
+// clamped LDS copy of expert_offset (unused when `grouped` is false: one expert owns [0, R)).
+__device__ __forceinline__ void locate_tile(int lin, int gnx, int ntiles_m, int ntiles_n, bool grouped,
+                                            const int64_t *s_off, int E, int64_t R, int BM, MTile &mt, int &tile_n)
+{
+    int tile_m;
+    if (gnx > 0) {
+        const int gm = 32 / gnx;
+        const int xcd = lin & 7, sl = (lin >> 3) & 31, round = lin >> 8;
+        const int rounds_n = (ntiles_n + 8 * gnx - 1) / (8 * gnx);
+        tile_m = (round / rounds_n) * gm + sl % gm;
+        tile_n = (round % rounds_n) * (8 * gnx) + xcd * gnx + sl / gm;
+    } else {
+        tile_m = lin / ntiles_n;
+        tile_n = lin % ntiles_n;
+    }
+    mt.e = 0;
+    mt.rows = 0;
+    mt.row0 = 0;
+    if (tile_m >= ntiles_m || tile_n >= ntiles_n) return;
+    if (!grouped) {
+        mt.row0 = static_cast<int64_t>(tile_m) * BM;
+        const int64_t left = R - mt.row0;
+        mt.rows = left <= 0 ? 0 : static_cast<int>(left < BM ? left : BM);
+        return;
+    }
+    int64_t tile = tile_m, prev = s_off[0];
+    for (int e = 0; e < E; ++e) {
+        int64_t hi = s_off[e + 1];
+        if (hi < prev) hi = prev;
+        const int64_t nt = (hi - prev + BM - 1) / BM;
+        if (tile < nt) {
+            // block-uniform by construction; say so to the compiler (scalar registers)
+            const int64_t row0 = prev + tile * BM, left = hi - row0;
+            mt.e = __builtin_amdgcn_readfirstlane(e);
+            mt.row0 = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0 >> 32))) << 32) |
+                      static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0)));
+            mt.rows = __builtin_amdgcn_readfirstlane(static_cast<int>(left < BM ? left : BM));
+            return;
+        }
+        tile -= nt;
+        prev = hi;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Persistent form of the direct-to-LDS kernel: one workgroup per CU walks the tile list
+// (linear tile id = blockIdx.x + i*gridDim.x, same XCD-grouped order as above) and the
+// k-tile pipeline runs straight through tile boundaries: while the last two k-tiles of a
+// tile are multiplied, the first two of the NEXT tile are already being loaded and its first
+// fragments read, so a tile costs no launch, no exposed first-load latency and no pipeline
+// refill; the output stores of one tile drain while the next one computes.
+// Requires K >= 128.  The wave that finds no further tile re-loads its current tile as the
+// "next" one (nobody reads it), which keeps the loop free of special cases.
+template <typename T, int BM, int BN, int WM, int WN, bool SWIGLU, bool ASM>
+__global__ __launch_bounds__(WM *WN * 64) void gemm_tiled16_persist_kernel(const T *__restrict__ X,
+                                                                            const int64_t *__restrict__ off,
+                                                                            const T *__restrict__ W,
+                                                                            const T *__restrict__ Bias, int E,
+                                                                            int64_t R, int64_t K, int64_t N,
+                                                                            T *__restrict__ Y, int ntiles_m,
+                                                                            int ntiles_n, int gnx, int total_lin)
+{
+    constexpr int NW = WM * WN;
+    constexpr int WTM = BM / WM, WTN = BN / WN, TMS = WTM / 16, TNS = WTN / 16, HM = TMS / 2;
+    constexpr int BNO = SWIGLU ? BN / 2 : BN;
+    constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW;   // 1 KiB wave loads per wave per k-tile
+    constexpr int NL = LA + LB, NLH = NL / 2, NM = HM * TNS;
+    constexpr int STAGE = (BM + BN) * ROWB;
+    static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0 && NL % 2 == 0, "tile/waves mismatch");
+    static_assert(HM + TNS + NLH <= NM, "not enough MFMA slots in a group for its memory instructions");
+    static_assert(!SWIGLU || TNS % 2 == 0, "SwiGLU needs an even number of n sub-tiles per wave");
+    using frag = typename Mfma<T>::frag;
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    __shared__ int64_t s_off[OPMX_MOE_MAX_EXPERTS + 1];
+
+    const int64_t ncols = SWIGLU ? N / 2 : N;
+    zero_unowned_rows(Y, R, ncols, off, E);
+    if (off != nullptr) {      // clamped copy of expert_offset, once per workgroup
+        for (int i = threadIdx.x; i <= E; i += blockDim.x) {
+            const int64_t v = off[i];
+            s_off[i] = v < 0 ? 0 : (v > R ? R : v);
+        }
+        __syncthreads();
+    }
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int lrow8 = lane >> 3, slot = lane & 7;
+
+    auto locate = [&](int lin, MTile &mt, int &tile_n) {
+        locate_tile(lin, gnx, ntiles_m, ntiles_n, off != nullptr, s_off, E, R, BM, mt, tile_n);
+    };
+    // first id >= lin (stepping by the grid size) that names work; total_lin if none
+    auto next_work = [&](int lin, MTile &mt, int &tile_n) {
+        for (; lin < total_lin; lin += gridDim.x) {
+            locate(lin, mt, tile_n);
+            if (mt.rows > 0) return lin;
+        }
+        mt.rows = 0;
+        return total_lin;
+    };
+    // this lane's global source offsets for a tile (bytes from the tile's X / W base at k = 0)
+    auto sources = [&](const MTile &mt, int tile_n, uint32_t (&a_src)[LA], uint32_t (&b_src)[LB]) {
+        const int64_t n0 = static_cast<int64_t>(tile_n) * BNO;
+#pragma unroll
+        for (int i = 0; i < LA; ++i) {
+            const int row = (wave * LA + i) * 8 + lrow8;
+            const int r = row < mt.rows ? row : mt.rows - 1;
+            const int c = slot ^ ((row >> 1) & 7);
+            a_src[i] = static_cast<uint32_t>((r * K + c * 8) * 2);
+        }
+#pragma unroll
+        for (int i = 0; i < LB; ++i) {
+            const int row = (wave * LB + i) * 8 + lrow8;
+            int64_t wrow;
+            if (SWIGLU) {
+                const int w = row / WTN, jj = row % WTN, half = jj / (WTN / 2);
+                int64_t ii = n0 + w * (WTN / 2) + jj % (WTN / 2);
+                ii = ii < ncols ? ii : ncols - 1;
+                wrow = half * ncols + ii;
+            } else {
+                wrow = n0 + row < N ? n0 + row : N - 1;
+            }
+            const int c = slot ^ ((row >> 1) & 7);
+            b_src[i] = static_cast<uint32_t>((wrow * K + c * 8) * 2);
+        }
+    };
+
+    MTile mt_c, mt_n;
+    int tn_c, tn_n;
+    int lin = next_work(blockIdx.x, mt_c, tn_c);
+    if (lin >= total_lin) return;
+    uint32_t asrc_c[LA], bsrc_c[LB], asrc_n[LA], bsrc_n[LB];
+    sources(mt_c, tn_c, asrc_c, bsrc_c);
+    // Buffer descriptors of a tile's X rows and of its expert's W matrix: the loads then take a
+    // scalar base, a scalar k offset and a 32-bit lane offset, i.e. no per-load address math.
+    __amdgpu_buffer_rsrc_t rx_c = raw_descriptor(X + mt_c.row0 * K);
+    __amdgpu_buffer_rsrc_t rw_c = raw_descriptor(W + static_cast<int64_t>(mt_c.e) * N * K);
+    __amdgpu_buffer_rsrc_t rx_n = rx_c, rw_n = rw_c;
+    const int a_lds = wave * LA * 1024, b_lds = BM * ROWB + wave * LB * 1024;   // wave-uniform
+
+    const int nk = static_cast<int>(K / BK);
+    const int lrow = lane & 15, lk = lane >> 4;
+    const int swz = (lrow >> 1) & 7;
+    const int x_off = (wm * WTM + lrow) * ROWB;
+    const int w_off = BM * ROWB + (wn * WTN + lrow) * ROWB;
+    const int co0 = ((lk ^ swz) << 4), co1 = (((4 + lk) ^ swz) << 4);
+    frag xf[2][HM], wf[2][TNS];
+    float4_t acc[TNS][TMS];
+
+    // wave load Q of k-tile KT of tile SET (c: current, n: next) into buffer BUF
+#define OPMX_ISSUE1(SET, KT, BUF, Q)                                                               \
+    do {                                                                                           \
+        char *st_ = smem + (BUF)*STAGE;                                                            \
+        const int kb_ = (KT)*ROWB;                                                                 \
+        if ((Q) < LA)                                                                              \
+            load_to_lds_16(rx_##SET, st_ + a_lds + (Q)*1024, asrc_##SET[(Q) < LA ? (Q) : 0], kb_); \
+        else                                                                                       \
+            load_to_lds_16(rw_##SET, st_ + b_lds + ((Q)-LA) * 1024, bsrc_##SET[(Q) < LA ? 0 : (Q)-LA], kb_); \
+    } while (0)
+#define OPMX_FRAG1(BUF, G, F)                                                                      \
+    do {                                                                                           \
+        const char *src_ = smem + (BUF)*STAGE + (((G) >> 1) ? co1 : co0);                          \
+        if (((G)&1) != 0)                                                                          \
+            xf[1][(F) < HM ? (F) : 0] = *reinterpret_cast<const frag *>(src_ + x_off + (HM + (F)) * 16 * ROWB); \
+        else if ((F) < HM)                                                                         \
+            xf[0][(F) < HM ? (F) : 0] = *reinterpret_cast<const frag *>(src_ + x_off + (F)*16 * ROWB); \
+        else                                                                                       \
+            wf[((G) >> 1) & 1][(F) < HM ? 0 : (F)-HM] =                                            \
+                *reinterpret_cast<const frag *>(src_ + w_off + ((F)-HM) * 16 * ROWB);              \
+    } while (0)
+#define OPMX_NFRAG(G) ((((G)&1) != 0) ? HM : HM + TNS)
+    // MFMA group G: MFMA m, then one fragment read of group G+1 (NREAD of them, buffer FBUF),
+    // then one wave load (numbers LQ0 .. LQ0+NLOAD-1 of k-tile LKT of tile SET into buffer LBUF)
+#define OPMX_GROUP(G, FBUF, NREAD, SET, LKT, LBUF, LQ0, NLOAD)                                     \
+    do {                                                                                           \
+        _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
+            if (ASM)                                                                               \
+                Mfma<T>::m16_acc(wf[((G) >> 1) & 1][m % TNS], xf[(G)&1][m / TNS],                  \
+                                 acc[m % TNS][((G)&1) * HM + m / TNS]);                            \
+            else                                                                                   \
+                acc[m % TNS][((G)&1) * HM + m / TNS] =                                             \
+                    Mfma<T>::m16(wf[((G) >> 1) & 1][m % TNS], xf[(G)&1][m / TNS],                  \
+                                 acc[m % TNS][((G)&1) * HM + m / TNS]);                            \
+            if (m < (NREAD)) OPMX_FRAG1(FBUF, ((G) + 1) & 3, m);                                   \
+            else if (m - (NREAD) < (NLOAD)) OPMX_ISSUE1(SET, LKT, LBUF, (LQ0) + m - (NREAD));      \
+        }                                                                                          \
+        if (!ASM) {                                                                                \
+            _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                       \
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                 \
+                if (m < (NREAD)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                \
+                else if (m - (NREAD) < (NLOAD)) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0); \
+            }                                                                                      \
+        }                                                                                          \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+    } while (0)
+    // One k-tile, read from buffer B.  Group 0 issues the second half of the loads of k-tile
+    // KT1 of tile SET1 into buffer B^1; after the barrier group 3 reads the first fragments from
+    // buffer B^1 and issues the first half of the loads of k-tile KT2 of tile SET2 into buffer B.
+#define OPMX_ITER(B, SET1, KT1, SET2, KT2)                                                         \
+    do {                                                                                           \
+        OPMX_GROUP(0, B, OPMX_NFRAG(1), SET1, KT1, (B) ^ 1, NLH, NL - NLH);                        \
+        OPMX_GROUP(1, B, OPMX_NFRAG(2), c, 0, 0, 0, 0);                                            \
+        OPMX_GROUP(2, B, OPMX_NFRAG(3), c, 0, 0, 0, 0);                                            \
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                           \
+        barrier_no_fence();                                                                        \
+        OPMX_GROUP(3, (B) ^ 1, OPMX_NFRAG(0), SET2, KT2, B, 0, NLH);                               \
+    } while (0)
+
+    // prologue of the first tile: k-tile 0 -> buffer 0, first half of k-tile 1 -> buffer 1
+#pragma unroll
+    for (int q = 0; q < NL; ++q) OPMX_ISSUE1(c, 0, 0, q);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    barrier_no_fence();
+#pragma unroll
+    for (int q = 0; q < NLH; ++q) OPMX_ISSUE1(c, 1, 1, q);
+#pragma unroll
+    for (int f = 0; f < HM + TNS; ++f) OPMX_FRAG1(0, 0, f);
+
+    int buf = 0;       // LDS buffer of the k-tile about to be multiplied
+    while (true) {
+        // the tile after this one (or this one again when the list is exhausted: a dummy
+        // whose loads land in buffers nobody reads)
+        const int lin_n = next_work(lin + gridDim.x, mt_n, tn_n);
+        const bool more = lin_n < total_lin;
+        if (!more) {
+            mt_n = mt_c;
+            tn_n = tn_c;
+        }
+        sources(mt_n, tn_n, asrc_n, bsrc_n);
+        rx_n = raw_descriptor(X + mt_n.row0 * K);
+        rw_n = raw_descriptor(W + static_cast<int64_t>(mt_n.e) * N * K);
+
+#pragma unroll
+        for (int j = 0; j < TNS; ++j)
+#pragma unroll
+            for (int i = 0; i < TMS; ++i)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc[j][i][v] = 0.0f;
+
+        int kt = 0;
+        for (; kt + 2 < nk; ++kt) {
+            OPMX_ITER(buf, c, kt + 1, c, kt + 2);
+            buf ^= 1;
+        }
+        OPMX_ITER(buf, c, kt + 1, n, 0);     // k-tile nk-2
+        buf ^= 1;
+        OPMX_ITER(buf, n, 0, n, 1);          // k-tile nk-1
+        buf ^= 1;
+
+        // asm MFMAs are opaque to the compiler's hazard padding: let the last ones retire
+        if (ASM) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+        tile_epilogue<T, WTM, WTN, SWIGLU>(acc, Bias, Y, mt_c, N, ncols, static_cast<int64_t>(tn_c) * BNO, wm, wn,
+                                           lane);
+        if (!more) break;
+        lin = lin_n;
+        mt_c = mt_n;
+        tn_c = tn_n;
+        rx_c = rx_n;
+        rw_c = rw_n;
+#pragma unroll
+        for (int i = 0; i < LA; ++i) asrc_c[i] = asrc_n[i];
+#pragma unroll
+        for (int i = 0; i < LB; ++i) bsrc_c[i] = bsrc_n[i];
+    }
+    // the dummy loads of the last tile must not outlive the workgroup's LDS allocation
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#undef OPMX_ITER
+#undef OPMX_GROUP
+#undef OPMX_NFRAG
+#undef OPMX_FRAG1
+#undef OPMX_ISSUE1
+}
+
+template <typename T, int BM, int BN, int WM, int WN>
+int tiled16_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
+                   int64_t N, int epilogue, void *Y, hipStream_t s)
+{
+    constexpr int smem = 2 * (BM + BN) * ROWB;
+    const bool sw = epilogue == OPMX_EPILOGUE_SWIGLU;
+    const int64_t ncols = sw ? N / 2 : N;
+    const int ntiles_n = static_cast<int>(ceil_div(ncols, sw ? BN / 2 : BN));
+    const int ntiles_m = static_cast<int>(max_mtiles(R, E, BM));
+    // XCD-grouped order only when the n-tiles split evenly over the 8 XCDs (else some XCDs idle)
+    int gnx = ntiles_n % 16 == 0 ? 2 : (ntiles_n % 8 == 0 ? 1 : 0);
+    if (const char *v = std::getenv("OPMX_MOE_GEMM_GNX")) gnx = std::atoi(v);   // tuning knob (0: row-major)
+    if (gnx != 0 && gnx != 1 && gnx != 2 && gnx != 4 && gnx != 8 && gnx != 16 && gnx != 32) gnx = 0;
+    const int64_t nblocks = gnx > 0 ? ceil_div(ntiles_n, 8 * gnx) * ceil_div(ntiles_m, 32 / gnx) * 256
+                                    : static_cast<int64_t>(ntiles_n) * ntiles_m;
+    dim3 grid(static_cast<unsigned>(nblocks));
+    dim3 block(WM * WN * 64);
+    static bool attr_done[2] = {false, false};
+    if (sw) {
+        auto kern = gemm_tiled16_kernel<T, BM, BN, WM, WN, true>;
+        if (!attr_done[1]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    smem) != hipSuccess)
+                return OPMX_ERR_LAUNCH;
+            attr_done[1] = true;
+        }
+        kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_m, ntiles_n, gnx);
+    } else {
+        auto kern = gemm_tiled16_kernel<T, BM, BN, WM, WN, false>;
+        if (!attr_done[0]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    smem) != hipSuccess)
+                return OPMX_ERR_LAUNCH;
+            attr_done[0] = true;
+        }
+        kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_m, ntiles_n, gnx);
+    }
+    OPMX_LAUNCH_CHECK();
+    return OPMX_OK;
+}
+
+template <typename T, int BM, int BN, int WM, int WN>
+int tiled16_dlds_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
+                        int64_t K, int64_t N, int epilogue, void *Y, hipStream_t s)
+{
+    constexpr int smem = 2 * (BM + BN) * ROWB;
+    constexpr bool ASM = (BM / WM) * (BN / WN) / 64 >= 256;   // 256 accumulator registers per lane
+    const bool sw = epilogue == OPMX_EPILOGUE_SWIGLU;
+    const int64_t ncols = sw ? N / 2 : N;
+    const int ntiles_n = static_cast<int>(ceil_div(ncols, sw ? BN / 2 : BN));
+    const int ntiles_m = static_cast<int>(max_mtiles(R, E, BM));
+    int gnx = ntiles_n % 16 == 0 ? 2 : (ntiles_n % 8 == 0 ? 1 : 0);
+    if (const char *v = std::getenv("OPMX_MOE_GEMM_GNX")) gnx = std::atoi(v);   // tuning knob (0: row-major)
+    if (gnx != 0 && gnx != 1 && gnx != 2 && gnx != 4 && gnx != 8 && gnx != 16 && gnx != 32) gnx = 0;
+    const int64_t nblocks = gnx > 0 ? ceil_div(ntiles_n, 8 * gnx) * ceil_div(ntiles_m, 32 / gnx) * 256
+                                    : static_cast<int64_t>(ntiles_n) * ntiles_m;
+    dim3 grid(static_cast<unsigned>(nblocks));
+    dim3 block(WM * WN * 64);
+    static bool attr_done[2] = {false, false};
+    if (sw) {
+        auto kern = gemm_tiled16_dlds_kernel<T, BM, BN, WM, WN, true, ASM>;
+        if (!attr_done[1]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    smem) != hipSuccess)
+                return OPMX_ERR_LAUNCH;
+            attr_done[1] = true;
+        }
+        kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_m, ntiles_n, gnx);
+    } else {
+        auto kern = gemm_tiled16_dlds_kernel<T, BM, BN, WM, WN, false, ASM>;
+        if (!attr_done[0]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    smem) != hipSuccess)
+                return OPMX_ERR_LAUNCH;
+            attr_done[0] = true;
+        }
+        kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_m, ntiles_n, gnx);
+    }
+    OPMX_LAUNCH_CHECK();
+    return OPMX_OK;
+}
+
+template <typename T, int BM, int BN, int WM, int WN>
+int tiled16_persist_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
+                           int64_t K, int64_t N, int epilogue, void *Y, hipStream_t s)
+{
+    constexpr int smem = 2 * (BM + BN) * ROWB;
+    constexpr bool ASM = (BM / WM) * (BN / WN) / 64 >= 256;   // 256 accumulator registers per lane
+    if (K < 2 * BK) return OPMX_ERR_UNSUPPORTED;
+    const bool sw = epilogue == OPMX_EPILOGUE_SWIGLU;
+    const int64_t ncols = sw ? N / 2 : N;
+    const int ntiles_n = static_cast<int>(ceil_div(ncols, sw ? BN / 2 : BN));
+    const int ntiles_m = static_cast<int>(max_mtiles(R, E, BM));
+    int gnx = ntiles_n % 16 == 0 ? 2 : (ntiles_n % 8 == 0 ? 1 : 0);
+    if (const char *v = std::getenv("OPMX_MOE_GEMM_GNX")) gnx = std::atoi(v);   // tuning knob (0: row-major)
+    if (gnx != 0 && gnx != 1 && gnx != 2 && gnx != 4 && gnx != 8 && gnx != 16 && gnx != 32) gnx = 0;
+    const int64_t total = gnx > 0 ? ceil_div(ntiles_n, 8 * gnx) * ceil_div(ntiles_m, 32 / gnx) * 256
+                                  : static_cast<int64_t>(ntiles_n) * ntiles_m;
+    if (total >= (int64_t{1} << 31)) return OPMX_ERR_UNSUPPORTED;
+    static int num_cu = 0;          // one workgroup per CU (its LDS footprint allows no second one)
+    if (num_cu == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            return OPMX_ERR_LAUNCH;
+        num_cu = n;
+    }
+    dim3 grid(static_cast<unsigned>(total < num_cu ? total : num_cu));
+    dim3 block(WM * WN * 64);
+    static bool attr_done[2] = {false, false};
+    if (sw) {
+        auto kern = gemm_tiled16_persist_kernel<T, BM, BN, WM, WN, true, ASM>;
+        if (!attr_done[1]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    smem) != hipSuccess)
+                return OPMX_ERR_LAUNCH;
+            attr_done[1] = true;
+        }
+        kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_m, ntiles_n, gnx,
+                                       static_cast<int>(total));
+    } else {
+        auto kern = gemm_tiled16_persist_kernel<T, BM, BN, WM, WN, false, ASM>;
+        if (!attr_done[0]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    smem) != hipSuccess)
+                return OPMX_ERR_LAUNCH;
+            attr_done[0] = true;
+        }
+        kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_m, ntiles_n, gnx,
+                                       static_cast<int>(total));
+    }
+    OPMX_LAUNCH_CHECK();
+    return OPMX_OK;
+}
+
+template <typename T>
+int tiled16_impl(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
+                 int64_t N, int epilogue, int variant, void *Y, hipStream_t s)
+{
+    switch (variant) {
+        case 1: return tiled16_launch<T, 256, 256, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        case 2: return tiled16_launch<T, 128, 128, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        case 3: return tiled16_dlds_launch<T, 256, 256, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        case 4: return tiled16_dlds_launch<T, 256, 256, 2, 4>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        // the persistent kernels pipeline across tiles and need at least two k-tiles
+        case 5:
+            if (K < 2 * BK) return tiled16_dlds_launch<T, 256, 256, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+            return tiled16_persist_launch<T, 256, 256, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        case 6:
+            if (K < 2 * BK) return tiled16_dlds_launch<T, 256, 256, 2, 4>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+            return tiled16_persist_launch<T, 256, 256, 2, 4>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        default: return tiled16_launch<T, 256, 256, 2, 4>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+    }
+}
+
+}  // namespace
+
+// Requires: dtype f16/bf16, K % 64 == 0, 16-byte aligned X and W, N*K < 2^31.
+int launch_gemm_tiled16(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
+                        int64_t K, int64_t N, int dtype, int epilogue, int variant, void *Y, hipStream_t s)
+{
+    switch (dtype) {
+        case OPMX_DTYPE_F16: return tiled16_impl<f16>(X, off, W, B, E, R, K, N, epilogue, variant, Y, s);
+        case OPMX_DTYPE_BF16: return tiled16_impl<bf16>(X, off, W, B, E, R, K, N, epilogue, variant, Y, s);
+    }
+    return OPMX_ERR_UNSUPPORTED;
+}
+
+}  // namespace opmx

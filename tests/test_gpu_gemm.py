@@ -83,7 +83,7 @@ def test_tiny_config_fp32_shapes():
     run_case("column", sizes, 1024, 5632, torch.float32, True, swiglu=True)
 
 
-@pytest.mark.parametrize("variant", ["0", "1", "2", "3", "4", "5", "6"])
+@pytest.mark.parametrize("variant", ["0", "1", "2", "3", "4", "5", "6", "7", "8", "9", "10", "11", "12", "13"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_tiled_kernel_variants(variant, dtype):
     env = {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": variant}
