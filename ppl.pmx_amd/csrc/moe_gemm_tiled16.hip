@@ -31,6 +31,127 @@ constexpr int CH = ROWB / 16;          // 16-byte chunks per row (8)
 // column land in sixteen different 16-byte bank groups (conflict-free b128 fragment reads).
 __device__ __forceinline__ int lds_off(int row, int chunk) { return row * ROWB + ((chunk ^ ((row >> 1) & 7)) << 4); }
 
+// Clamped copy of expert_offset in LDS (values forced into a non-decreasing sequence inside
+// [0, R] when read, so a corrupt offset can never send a store outside Y).  Nothing to do for a
+// dense GEMM (off == nullptr).  Every thread must call it: it contains a block barrier.
+__device__ __forceinline__ void stage_offsets(const int64_t *__restrict__ off, int E, int64_t R, int64_t *s_off)
+{
+    if (off == nullptr) return;
+    for (int i = threadIdx.x; i <= E; i += blockDim.x) {
+        const int64_t v = off[i];
+        s_off[i] = v < 0 ? 0 : (v > R ? R : v);
+    }
+    __syncthreads();
+}
+
+// Number of row tiles of height BM over all experts: sum of ceil(rows_e / BM).
+__device__ __forceinline__ int count_mtiles(bool grouped, const int64_t *s_off, int E, int64_t R, int BM)
+{
+    if (!grouped) return static_cast<int>((R + BM - 1) / BM);
+    int64_t total = 0, prev = s_off[0];
+    for (int e = 0; e < E; ++e) {
+        int64_t hi = s_off[e + 1];
+        if (hi < prev) hi = prev;
+        total += (hi - prev + BM - 1) / BM;
+        prev = hi;
+    }
+    return __builtin_amdgcn_readfirstlane(static_cast<int>(total));
+}
+
+// Linear tile id -> (row tile, column tile); mtiles is the actual number of row tiles.
+// Workgroups are handed to the 8 XCDs round-robin by linear id and each XCD has its own L2, so
+// 256 consecutive ids ("a round", 32 per XCD) form a block of tiles in which every XCD owns a
+// compact sub-block: its 32 resident workgroups then share X- and W-tiles in that XCD's L2.
+//   gnx = 1, 2: XCDs side by side along n, each (32/gnx) x gnx tiles;
+//   gnx = 4   : rounds of 16 x 16 tiles, XCDs as 2 (m) x 4 (n), each 8 x 4 tiles (a third less
+//               L2 fill traffic than 16 x 2).  The last mtiles % 16 row tiles would leave XCDs
+//               idle in that layout; they are dealt out differently: XCD j takes the column
+//               tiles [j*ntiles_n/8, (j+1)*ntiles_n/8), walking m fastest.  ntiles_n % 16 == 0.
+//   gnx = 0   : plain row-major order, n fastest.
+// Ids that name no tile come back with tile_m >= mtiles.
+__device__ __forceinline__ void map_tile(int lin, int gnx, int mtiles, int ntiles_n, int &tile_m, int &tile_n)
+{
+    const int xcd = lin & 7, sl = (lin >> 3) & 31, round = lin >> 8;
+    if (gnx == 4) {
+        const int cols16 = ntiles_n / 16, full = mtiles / 16, rem = mtiles % 16;
+        const int ids_full = full * cols16 * 256;
+        if (lin < ids_full) {
+            tile_m = (round / cols16) * 16 + (xcd >> 2) * 8 + (sl & 7);
+            tile_n = (round % cols16) * 16 + (xcd & 3) * 4 + (sl >> 3);
+        } else {
+            const int s = (lin - ids_full) >> 3, cols = ntiles_n / 8;
+            if (rem > 0 && s < rem * cols) {
+                tile_m = full * 16 + s % rem;
+                tile_n = xcd * cols + s / rem;
+            } else {
+                tile_m = mtiles;
+                tile_n = 0;
+            }
+        }
+    } else if (gnx > 0) {
+        const int gm = 32 / gnx;
+        const int rounds_n = (ntiles_n + 8 * gnx - 1) / (8 * gnx);
+        tile_m = (round / rounds_n) * gm + sl % gm;
+        tile_n = (round % rounds_n) * (8 * gnx) + xcd * gnx + sl / gm;
+    } else {
+        tile_m = lin / ntiles_n;
+        tile_n = lin % ntiles_n;
+    }
+}
+
+// Linear tile id -> (row tile of one expert, column tile).  mt.rows == 0 when the id names no
+// work.  s_off: see stage_offsets (unused when `grouped` is false: one expert owns [0, R)).
+__device__ __forceinline__ void locate_tile(int lin, int gnx, int mtiles, int ntiles_n, bool grouped,
+                                            const int64_t *s_off, int E, int64_t R, int BM, MTile &mt, int &tile_n)
+{
+    int tile_m;
+    map_tile(lin, gnx, mtiles, ntiles_n, tile_m, tile_n);
+    mt.e = 0;
+    mt.rows = 0;
+    mt.row0 = 0;
+    if (tile_m >= mtiles || tile_n >= ntiles_n) return;
+    if (!grouped) {
+        mt.row0 = static_cast<int64_t>(tile_m) * BM;
+        const int64_t left = R - mt.row0;
+        mt.rows = left <= 0 ? 0 : static_cast<int>(left < BM ? left : BM);
+        return;
+    }
+    int64_t tile = tile_m, prev = s_off[0];
+    for (int e = 0; e < E; ++e) {
+        int64_t hi = s_off[e + 1];
+        if (hi < prev) hi = prev;
+        const int64_t nt = (hi - prev + BM - 1) / BM;
+        if (tile < nt) {
+            // block-uniform by construction; say so to the compiler (scalar registers)
+            const int64_t row0 = prev + tile * BM, left = hi - row0;
+            mt.e = __builtin_amdgcn_readfirstlane(e);
+            mt.row0 = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0 >> 32))) << 32) |
+                      static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0)));
+            mt.rows = __builtin_amdgcn_readfirstlane(static_cast<int>(left < BM ? left : BM));
+            return;
+        }
+        tile -= nt;
+        prev = hi;
+    }
+}
+
+// Host side of map_tile: the order to use and the number of linear ids it spans.
+inline int pick_gnx(int ntiles_n)
+{
+    // XCD-grouped orders only when the n-tiles split evenly over the rounds (else XCDs idle)
+    int gnx = ntiles_n % 16 == 0 ? 4 : (ntiles_n % 8 == 0 ? 1 : 0);
+    if (const char *v = std::getenv("OPMX_MOE_GEMM_GNX")) gnx = std::atoi(v);   // tuning knob
+    if (gnx != 0 && gnx != 1 && gnx != 2 && gnx != 4) gnx = 0;
+    if (gnx == 4 && ntiles_n % 16 != 0) gnx = 0;
+    return gnx;
+}
+inline int64_t linear_ids(int gnx, int ntiles_m, int ntiles_n)
+{
+    if (gnx == 4) return ceil_div(ntiles_n, 16) * ceil_div(ntiles_m, 16) * 256;
+    if (gnx > 0) return ceil_div(ntiles_n, 8 * gnx) * ceil_div(ntiles_m, 32 / gnx) * 256;
+    return static_cast<int64_t>(ntiles_n) * ntiles_m;
+}
+
 // Writes a wave's accumulators.  acc[j][i][v] is output row (X row) i*16 + lane%16 and output
 // column j*16 + (lane/16)*4 + v of the WTM x WTN wave tile: four consecutive columns per lane,
 // stored as one 8-byte word.  With SWIGLU sub-tiles j and j + TNS/2 hold gate and up columns.
@@ -104,22 +225,11 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled16_kernel(const T *__re
     const int64_t ncols = SWIGLU ? N / 2 : N;
     zero_unowned_rows(Y, R, ncols, off, E);
 
-    // Block -> tile map: 256 consecutive block ids (32 per XCD, ids go round-robin over the
-    // 8 XCDs) form a gm x (8*gnx) block of tiles in which XCD j owns a compact gm x gnx
-    // sub-block, so its resident blocks share X- and W-tiles in that XCD's L2.
-    int tile_m, tile_n;
-    if (gnx > 0) {
-        const int gm = 32 / gnx;
-        const int lin = blockIdx.x, xcd = lin & 7, slot = (lin >> 3) & 31, round = lin >> 8;
-        const int rounds_n = (ntiles_n + 8 * gnx - 1) / (8 * gnx);
-        tile_m = (round / rounds_n) * gm + slot % gm;
-        tile_n = (round % rounds_n) * (8 * gnx) + xcd * gnx + slot / gm;
-    } else {
-        tile_m = blockIdx.x / ntiles_n;
-        tile_n = blockIdx.x % ntiles_n;
-    }
-    if (tile_m >= ntiles_m || tile_n >= ntiles_n) return;
-    const MTile mt = find_mtile(off, E, R, BM, tile_m, s_off);
+    stage_offsets(off, E, R, s_off);
+    MTile mt;
+    int tile_n;
+    locate_tile(blockIdx.x, gnx, count_mtiles(off != nullptr, s_off, E, R, BM), ntiles_n, off != nullptr, s_off, E, R,
+                BM, mt, tile_n);
     if (mt.rows == 0) return;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -337,19 +447,11 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled16_dlds_kernel(const T 
 
     const int64_t ncols = SWIGLU ? N / 2 : N;
     zero_unowned_rows(Y, R, ncols, off, E);
-    int tile_m, tile_n;
-    if (gnx > 0) {
-        const int gm = 32 / gnx;
-        const int lin = blockIdx.x, xcd = lin & 7, slot = (lin >> 3) & 31, round = lin >> 8;
-        const int rounds_n = (ntiles_n + 8 * gnx - 1) / (8 * gnx);
-        tile_m = (round / rounds_n) * gm + slot % gm;
-        tile_n = (round % rounds_n) * (8 * gnx) + xcd * gnx + slot / gm;
-    } else {
-        tile_m = blockIdx.x / ntiles_n;
-        tile_n = blockIdx.x % ntiles_n;
-    }
-    if (tile_m >= ntiles_m || tile_n >= ntiles_n) return;
-    const MTile mt = find_mtile(off, E, R, BM, tile_m, s_off);
+    stage_offsets(off, E, R, s_off);
+    MTile mt;
+    int tile_n;
+    locate_tile(blockIdx.x, gnx, count_mtiles(off != nullptr, s_off, E, R, BM), ntiles_n, off != nullptr, s_off, E, R,
+                BM, mt, tile_n);
     if (mt.rows == 0) return;
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -512,52 +614,6 @@ __device__ __forceinline__ void load_to_lds_16(__amdgpu_buffer_rsrc_t r, char *l
     __builtin_amdgcn_raw_ptr_buffer_load_lds(r, OPMX_LPTR(lds), 16, voff, soff, 0, 0);
 }
 
-// Linear tile id -> (row tile of one expert, column tile), in the XCD-grouped order described
-// at the tile map of the kernels above.  mt.rows == 0 when the id names no work.  s_off is the
-// clamped LDS copy of expert_offset (unused when `grouped` is false: one expert owns [0, R)).
-__device__ __forceinline__ void locate_tile(int lin, int gnx, int ntiles_m, int ntiles_n, bool grouped,
-                                            const int64_t *s_off, int E, int64_t R, int BM, MTile &mt, int &tile_n)
-{
-    int tile_m;
-    if (gnx > 0) {
-        const int gm = 32 / gnx;
-        const int xcd = lin & 7, sl = (lin >> 3) & 31, round = lin >> 8;
-        const int rounds_n = (ntiles_n + 8 * gnx - 1) / (8 * gnx);
-        tile_m = (round / rounds_n) * gm + sl % gm;
-        tile_n = (round % rounds_n) * (8 * gnx) + xcd * gnx + sl / gm;
-    } else {
-        tile_m = lin / ntiles_n;
-        tile_n = lin % ntiles_n;
-    }
-    mt.e = 0;
-    mt.rows = 0;
-    mt.row0 = 0;
-    if (tile_m >= ntiles_m || tile_n >= ntiles_n) return;
-    if (!grouped) {
-        mt.row0 = static_cast<int64_t>(tile_m) * BM;
-        const int64_t left = R - mt.row0;
-        mt.rows = left <= 0 ? 0 : static_cast<int>(left < BM ? left : BM);
-        return;
-    }
-    int64_t tile = tile_m, prev = s_off[0];
-    for (int e = 0; e < E; ++e) {
-        int64_t hi = s_off[e + 1];
-        if (hi < prev) hi = prev;
-        const int64_t nt = (hi - prev + BM - 1) / BM;
-        if (tile < nt) {
-            // block-uniform by construction; say so to the compiler (scalar registers)
-            const int64_t row0 = prev + tile * BM, left = hi - row0;
-            mt.e = __builtin_amdgcn_readfirstlane(e);
-            mt.row0 = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0 >> 32))) << 32) |
-                      static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0)));
-            mt.rows = __builtin_amdgcn_readfirstlane(static_cast<int>(left < BM ? left : BM));
-            return;
-        }
-        tile -= nt;
-        prev = hi;
-    }
-}
-
 // ---------------------------------------------------------------------------------------
 // Persistent form of the direct-to-LDS kernel: one workgroup per CU walks the tile list
 // (linear tile id = blockIdx.x + i*gridDim.x, same XCD-grouped order as above) and the
@@ -592,13 +648,8 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled16_persist_kernel(const
 
     const int64_t ncols = SWIGLU ? N / 2 : N;
     zero_unowned_rows(Y, R, ncols, off, E);
-    if (off != nullptr) {      // clamped copy of expert_offset, once per workgroup
-        for (int i = threadIdx.x; i <= E; i += blockDim.x) {
-            const int64_t v = off[i];
-            s_off[i] = v < 0 ? 0 : (v > R ? R : v);
-        }
-        __syncthreads();
-    }
+    stage_offsets(off, E, R, s_off);      // once per workgroup
+    const int mtiles = count_mtiles(off != nullptr, s_off, E, R, BM);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -606,7 +657,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled16_persist_kernel(const
     const int lrow8 = lane >> 3, slot = lane & 7;
 
     auto locate = [&](int lin, MTile &mt, int &tile_n) {
-        locate_tile(lin, gnx, ntiles_m, ntiles_n, off != nullptr, s_off, E, R, BM, mt, tile_n);
+        locate_tile(lin, gnx, mtiles, ntiles_n, off != nullptr, s_off, E, R, BM, mt, tile_n);
     };
     // first id >= lin (stepping by the grid size) that names work; total_lin if none
     auto next_work = [&](int lin, MTile &mt, int &tile_n) {
@@ -799,12 +850,8 @@ int tiled16_launch(const void *X, const int64_t *off, const void *W, const void 
     const int64_t ncols = sw ? N / 2 : N;
     const int ntiles_n = static_cast<int>(ceil_div(ncols, sw ? BN / 2 : BN));
     const int ntiles_m = static_cast<int>(max_mtiles(R, E, BM));
-    // XCD-grouped order only when the n-tiles split evenly over the 8 XCDs (else some XCDs idle)
-    int gnx = ntiles_n % 16 == 0 ? 2 : (ntiles_n % 8 == 0 ? 1 : 0);
-    if (const char *v = std::getenv("OPMX_MOE_GEMM_GNX")) gnx = std::atoi(v);   // tuning knob (0: row-major)
-    if (gnx != 0 && gnx != 1 && gnx != 2 && gnx != 4 && gnx != 8 && gnx != 16 && gnx != 32) gnx = 0;
-    const int64_t nblocks = gnx > 0 ? ceil_div(ntiles_n, 8 * gnx) * ceil_div(ntiles_m, 32 / gnx) * 256
-                                    : static_cast<int64_t>(ntiles_n) * ntiles_m;
+    const int gnx = pick_gnx(ntiles_n);
+    const int64_t nblocks = linear_ids(gnx, ntiles_m, ntiles_n);
     dim3 grid(static_cast<unsigned>(nblocks));
     dim3 block(WM * WN * 64);
     static bool attr_done[2] = {false, false};
@@ -843,11 +890,8 @@ int tiled16_dlds_launch(const void *X, const int64_t *off, const void *W, const 
     const int64_t ncols = sw ? N / 2 : N;
     const int ntiles_n = static_cast<int>(ceil_div(ncols, sw ? BN / 2 : BN));
     const int ntiles_m = static_cast<int>(max_mtiles(R, E, BM));
-    int gnx = ntiles_n % 16 == 0 ? 2 : (ntiles_n % 8 == 0 ? 1 : 0);
-    if (const char *v = std::getenv("OPMX_MOE_GEMM_GNX")) gnx = std::atoi(v);   // tuning knob (0: row-major)
-    if (gnx != 0 && gnx != 1 && gnx != 2 && gnx != 4 && gnx != 8 && gnx != 16 && gnx != 32) gnx = 0;
-    const int64_t nblocks = gnx > 0 ? ceil_div(ntiles_n, 8 * gnx) * ceil_div(ntiles_m, 32 / gnx) * 256
-                                    : static_cast<int64_t>(ntiles_n) * ntiles_m;
+    const int gnx = pick_gnx(ntiles_n);
+    const int64_t nblocks = linear_ids(gnx, ntiles_m, ntiles_n);
     dim3 grid(static_cast<unsigned>(nblocks));
     dim3 block(WM * WN * 64);
     static bool attr_done[2] = {false, false};
@@ -887,11 +931,8 @@ int tiled16_persist_launch(const void *X, const int64_t *off, const void *W, con
     const int64_t ncols = sw ? N / 2 : N;
     const int ntiles_n = static_cast<int>(ceil_div(ncols, sw ? BN / 2 : BN));
     const int ntiles_m = static_cast<int>(max_mtiles(R, E, BM));
-    int gnx = ntiles_n % 16 == 0 ? 2 : (ntiles_n % 8 == 0 ? 1 : 0);
-    if (const char *v = std::getenv("OPMX_MOE_GEMM_GNX")) gnx = std::atoi(v);   // tuning knob (0: row-major)
-    if (gnx != 0 && gnx != 1 && gnx != 2 && gnx != 4 && gnx != 8 && gnx != 16 && gnx != 32) gnx = 0;
-    const int64_t total = gnx > 0 ? ceil_div(ntiles_n, 8 * gnx) * ceil_div(ntiles_m, 32 / gnx) * 256
-                                  : static_cast<int64_t>(ntiles_n) * ntiles_m;
+    const int gnx = pick_gnx(ntiles_n);
+    const int64_t total = linear_ids(gnx, ntiles_m, ntiles_n);
     if (total >= (int64_t{1} << 31)) return OPMX_ERR_UNSUPPORTED;
     static int num_cu = 0;          // one workgroup per CU (its LDS footprint allows no second one)
     if (num_cu == 0) {

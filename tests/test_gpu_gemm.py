@@ -95,6 +95,17 @@ def test_tiled_kernel_variants(variant, dtype):
     run_case("column", sizes, 64, 1000, dtype, False, env, swiglu=True)   # D=500: ragged epilogue tile
 
 
+@pytest.mark.parametrize("variant", ["7", "10", "11", "12", "13"])
+def test_tile_order_with_partial_last_round(variant):
+    """16 column tiles and 24 row tiles: one full 16 x 16 round in the XCD-grouped order plus
+    eight row tiles dealt out by the remainder rule; SwiGLU case: 16 column tiles of 128."""
+    env = {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": variant}
+    sizes = [1500, 0, 700, 33, 1281, 256, 5, 1300]
+    run_case("column", sizes, 128, 4096, torch.float16, True, env)
+    run_case("column", sizes, 128, 4096, torch.bfloat16, False, env, swiglu=True)
+    run_case("row", [4096], 192, 4096, torch.float16, False, env)          # exactly one full round
+
+
 @pytest.mark.parametrize("variant", ["0", "1", "2", "3", "4", "5"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_stream_kernel_variants(variant, dtype):
