@@ -198,6 +198,57 @@ __device__ __forceinline__ void tile_epilogue(float4_t (&acc)[WTN / 16][WTM / 16
     }
 }
 
+// Same result as tile_epilogue, but staged through a wave-private LDS region (WTM rows of the
+// wave's output columns, 16-byte chunks XOR-swizzled by row) so that global memory sees whole
+// rows of the wave tile: each store instruction writes 1 KiB as runs of 128/256 contiguous
+// bytes instead of 32-byte pieces.  No block barrier is needed (a wave only touches its own
+// region, and its LDS operations execute in order); the caller guarantees that no wave still
+// reads operand tiles from LDS.  Requires ncols % 8 == 0 and a 16-byte aligned Y.
+template <typename T, int WTM, int WTN, bool SWIGLU>
+__device__ __forceinline__ void tile_epilogue_lds(float4_t (&acc)[WTN / 16][WTM / 16], const T *__restrict__ Bias,
+                                                  T *__restrict__ Y, const MTile &mt, int64_t N, int64_t ncols,
+                                                  int64_t n0, int wm, int wn, int lane, char *wave_lds)
+{
+    constexpr int TMS = WTM / 16, TNS = WTN / 16, NO = SWIGLU ? TNS / 2 : TNS;
+    constexpr int ROWP = NO * 16 * 2;          // bytes per staged row
+    constexpr int CH16 = ROWP / 16;            // 16-byte chunks per staged row
+    constexpr int RPI = 1024 / ROWP;           // rows per wave-wide 16-byte access
+    const int lrow = lane & 15, lk = lane >> 4;
+    const T *be = Bias ? Bias + static_cast<int64_t>(mt.e) * N : nullptr;
+    const int64_t nw0 = (SWIGLU ? n0 + wn * (WTN / 2) : n0 + wn * WTN);   // first output column of this wave
+#pragma unroll
+    for (int i = 0; i < TMS; ++i) {
+        const int row = i * 16 + lrow;
+#pragma unroll
+        for (int j = 0; j < NO; ++j) {
+            const int64_t n = nw0 + j * 16 + lk * 4;
+            T out[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int64_t nn = n + v < ncols ? n + v : ncols - 1;
+                float g = acc[j][i][v] + (be ? to_f32(be[nn]) : 0.0f);
+                if (SWIGLU) {
+                    const float up = acc[j + TNS / 2][i][v] + (be ? to_f32(be[ncols + nn]) : 0.0f);
+                    g = up * g * sigmoidf_(g);
+                }
+                out[v] = from_f32<T>(g);
+            }
+            const int chunk = j * 2 + (lk >> 1);
+            *reinterpret_cast<uint2 *>(wave_lds + row * ROWP + ((chunk ^ (row % CH16)) << 4) + (lk & 1) * 8) =
+                *reinterpret_cast<const uint2 *>(out);
+        }
+    }
+#pragma unroll
+    for (int rr = 0; rr < WTM / RPI; ++rr) {
+        const int row = rr * RPI + lane / CH16, c = lane % CH16;
+        const u32x4 v = *reinterpret_cast<const u32x4 *>(wave_lds + row * ROWP + ((c ^ (row % CH16)) << 4));
+        const int grow = wm * WTM + row;
+        const int64_t n = nw0 + c * 8;
+        if (grow < mt.rows && n < ncols)       // ncols % 8 == 0: a chunk is inside or outside as a whole
+            *reinterpret_cast<u32x4 *>(Y + (mt.row0 + grow) * ncols + n) = v;
+    }
+}
+
 template <typename T, int BM, int BN, int WM, int WN, bool SWIGLU>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled16_kernel(const T *__restrict__ X,
                                                                     const int64_t *__restrict__ off,
@@ -615,6 +666,185 @@ __device__ __forceinline__ void load_to_lds_16(__amdgpu_buffer_rsrc_t r, char *l
 }
 
 // ---------------------------------------------------------------------------------------
+// Direct-to-LDS, 4 waves, fragments of a whole k-tile held in registers.  Each wave reads all
+// 32 fragments of k-tile kt (128 VGPRs) by the first third of the k-tile, so the LDS buffer is
+// free again a good k-tile before it is needed and the loads of k-tile kt+2 get more than a
+// whole k-tile to land behind MFMAs: the slowest load of the slowest wave, which every wave
+// waits for at the barrier, stops being the pace setter.  Two barriers per k-tile:
+//   A (group 1, after this wave's last fragment read of buffer kt&1 returned): buffer free ->
+//     16 loads of k-tile kt+2 into it, one every third MFMA of groups 1-2;
+//   B (before group 3, after s_waitcnt vmcnt(16): this wave's loads of k-tile kt+1 landed) ->
+//     group 3 reads the first fragments of k-tile kt+1.
+// MFMAs are volatile asm (accumulators pinned to the 256 accumulation registers), so the
+// source order below is the issue order.
+template <typename T, int BM, int BN, bool SWIGLU>
+__global__ __launch_bounds__(256) void gemm_tiled16_plr_kernel(const T *__restrict__ X,
+                                                               const int64_t *__restrict__ off,
+                                                               const T *__restrict__ W,
+                                                               const T *__restrict__ Bias, int E, int64_t R,
+                                                               int64_t K, int64_t N, T *__restrict__ Y,
+                                                               int ntiles_n, int gnx)
+{
+    constexpr int WM = 2, WN = 2, NW = 4;
+    constexpr int WTM = BM / WM, WTN = BN / WN, TMS = WTM / 16, TNS = WTN / 16, HM = TMS / 2;
+    constexpr int BNO = SWIGLU ? BN / 2 : BN;
+    constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW, NL = LA + LB;   // 1 KiB wave loads per k-tile
+    constexpr int STAGE = (BM + BN) * ROWB;
+    constexpr int NM = HM * TNS;
+    static_assert(HM == 4 && TNS == 8 && NL == 16, "the schedule below is written for 128x128 wave tiles");
+    using frag = typename Mfma<T>::frag;
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    __shared__ int64_t s_off[OPMX_MOE_MAX_EXPERTS + 1];
+
+    const int64_t ncols = SWIGLU ? N / 2 : N;
+    zero_unowned_rows(Y, R, ncols, off, E);
+    stage_offsets(off, E, R, s_off);
+    MTile mt;
+    int tile_n;
+    locate_tile(blockIdx.x, gnx, count_mtiles(off != nullptr, s_off, E, R, BM), ntiles_n, off != nullptr, s_off, E, R,
+                BM, mt, tile_n);
+    if (mt.rows == 0) return;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int64_t n0 = static_cast<int64_t>(tile_n) * BNO;
+    const __amdgpu_buffer_rsrc_t rx = raw_descriptor(X + mt.row0 * K);
+    const __amdgpu_buffer_rsrc_t rw = raw_descriptor(W + static_cast<int64_t>(mt.e) * N * K);
+
+    // this lane's share of the wave loads: tile row 8*(wave*L+i) + lane/8, LDS slot lane%8
+    const int lrow8 = lane >> 3, slot = lane & 7;
+    uint32_t a_src[LA], b_src[LB];     // byte offsets from the tile's X / W base at k = 0
+#pragma unroll
+    for (int i = 0; i < LA; ++i) {
+        const int row = (wave * LA + i) * 8 + lrow8;
+        const int r = row < mt.rows ? row : mt.rows - 1;
+        const int c = slot ^ ((row >> 1) & 7);
+        a_src[i] = static_cast<uint32_t>((r * K + c * 8) * 2);
+    }
+#pragma unroll
+    for (int i = 0; i < LB; ++i) {
+        const int row = (wave * LB + i) * 8 + lrow8;
+        int64_t wrow;
+        if (SWIGLU) {
+            const int w = row / WTN, jj = row % WTN, half = jj / (WTN / 2);
+            int64_t ii = n0 + w * (WTN / 2) + jj % (WTN / 2);
+            ii = ii < ncols ? ii : ncols - 1;
+            wrow = half * ncols + ii;
+        } else {
+            wrow = n0 + row < N ? n0 + row : N - 1;
+        }
+        const int c = slot ^ ((row >> 1) & 7);
+        b_src[i] = static_cast<uint32_t>((wrow * K + c * 8) * 2);
+    }
+    const int a_lds = wave * LA * 1024, b_lds = BM * ROWB + wave * LB * 1024;   // wave-uniform
+
+    float4_t acc[TNS][TMS];
+#pragma unroll
+    for (int j = 0; j < TNS; ++j)
+#pragma unroll
+        for (int i = 0; i < TMS; ++i)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[j][i][v] = 0.0f;
+
+    const int nk = static_cast<int>(K / BK);
+    const int lrow = lane & 15, lk = lane >> 4;
+    const int swz = (lrow >> 1) & 7;
+    const int x_off = (wm * WTM + lrow) * ROWB;
+    const int w_off = BM * ROWB + (wn * WTN + lrow) * ROWB;
+    const int co0 = ((lk ^ swz) << 4), co1 = (((4 + lk) ^ swz) << 4);
+    frag xf[2][2][HM], wf[2][TNS];      // [k32 step][X half][sub-tile], [k32 step][sub-tile]
+
+    // wave load Q of k-tile KT into buffer BUF: Q < LA -> X rows, else W rows
+#define OPMX_ISSUE1(KT, BUF, Q)                                                                    \
+    do {                                                                                           \
+        char *st_ = smem + (BUF)*STAGE;                                                            \
+        const int kb_ = (KT)*ROWB;                                                                 \
+        if ((Q) < LA) load_to_lds_16(rx, st_ + a_lds + (Q)*1024, a_src[(Q) < LA ? (Q) : 0], kb_);  \
+        else load_to_lds_16(rw, st_ + b_lds + ((Q)-LA) * 1024, b_src[(Q) < LA ? 0 : (Q)-LA], kb_); \
+    } while (0)
+#define OPMX_XFRAG(BUF, S, H, I)                                                                   \
+    xf[S][H][I] = *reinterpret_cast<const frag *>(smem + (BUF)*STAGE + ((S) ? co1 : co0) + x_off + ((H)*HM + (I)) * 16 * ROWB)
+#define OPMX_WFRAG(BUF, S, J)                                                                      \
+    wf[S][J] = *reinterpret_cast<const frag *>(smem + (BUF)*STAGE + ((S) ? co1 : co0) + w_off + (J)*16 * ROWB)
+#define OPMX_MF(S, H, m) Mfma<T>::m16_acc(wf[S][(m) % TNS], xf[S][H][(m) / TNS], acc[(m) % TNS][(H)*HM + (m) / TNS])
+    // k-tile in buffer B.  LD2: k-tile KT+2 exists (loaded into buffer B).  NEXT: k-tile KT+1 exists.
+#define OPMX_ITER(KT, B, LD2, NEXT)                                                                \
+    do {                                                                                           \
+        _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
+            OPMX_MF(0, 0, m);                                                                      \
+            if (m % 2 == 0) {                                                                      \
+                const int r = m / 2;                                                               \
+                if (r < 4) OPMX_XFRAG(B, 0, 1, r < 4 ? r : 0);                                     \
+                else if (r < 8) OPMX_XFRAG(B, 1, 0, (r >= 4 && r < 8) ? r - 4 : 0);                \
+                else OPMX_WFRAG(B, 1, r >= 8 ? r - 8 : 0);                                         \
+            }                                                                                      \
+        }                                                                                          \
+        _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
+            OPMX_MF(0, 1, m);                                                                      \
+            if (m < 4) OPMX_XFRAG(B, 1, 1, m < 4 ? m : 0);                                         \
+            if (m == 10) barrier_no_fence();                                                       \
+            if ((LD2) && m >= 11 && (m - 11) % 3 == 0) OPMX_ISSUE1((KT) + 2, B, (m - 11) / 3);     \
+        }                                                                                          \
+        _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
+            OPMX_MF(1, 0, m);                                                                      \
+            if ((LD2) && m % 3 == 0 && m / 3 < 9) OPMX_ISSUE1((KT) + 2, B, 7 + m / 3);             \
+        }                                                                                          \
+        if (LD2) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");                                 \
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                      \
+        __builtin_amdgcn_s_barrier();                                                              \
+        asm volatile("" ::: "memory");                                                             \
+        _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
+            OPMX_MF(1, 1, m);                                                                      \
+            if ((NEXT) && m < 4) OPMX_XFRAG((B) ^ 1, 0, 0, m < 4 ? m : 0);                         \
+            else if ((NEXT) && m < 12) OPMX_WFRAG((B) ^ 1, 0, (m >= 4 && m < 12) ? m - 4 : 0);     \
+        }                                                                                          \
+    } while (0)
+
+    // prologue: k-tile 0 -> buffer 0, k-tile 1 -> buffer 1, wait for k-tile 0
+#pragma unroll
+    for (int q = 0; q < NL; ++q) OPMX_ISSUE1(0, 0, q);
+    if (nk > 1) {
+#pragma unroll
+        for (int q = 0; q < NL; ++q) OPMX_ISSUE1(1, 1, q);
+        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < HM; ++i) OPMX_XFRAG(0, 0, 0, i);
+#pragma unroll
+    for (int j = 0; j < TNS; ++j) OPMX_WFRAG(0, 0, j);
+    {
+        int kt = 0, b = 0;
+        for (; kt + 2 < nk; ++kt, b ^= 1) OPMX_ITER(kt, b, true, true);
+        if (kt + 1 < nk) {
+            OPMX_ITER(kt, b, false, true);
+            ++kt;
+            b ^= 1;
+        }
+        OPMX_ITER(kt, b, false, false);
+    }
+#undef OPMX_ITER
+#undef OPMX_MF
+#undef OPMX_WFRAG
+#undef OPMX_XFRAG
+#undef OPMX_ISSUE1
+
+    // asm MFMAs are opaque to the compiler's hazard padding: let the last ones retire
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    // after the last barrier no wave reads operand tiles any more: LDS is free for the epilogue
+    if (ncols % 8 == 0 && reinterpret_cast<uintptr_t>(Y) % 16 == 0)
+        tile_epilogue_lds<T, WTM, WTN, SWIGLU>(acc, Bias, Y, mt, N, ncols, n0, wm, wn, lane,
+                                               smem + wave * (WTM * (SWIGLU ? WTN / 2 : WTN) * 2));
+    else
+        tile_epilogue<T, WTM, WTN, SWIGLU>(acc, Bias, Y, mt, N, ncols, n0, wm, wn, lane);
+}
+
+// ---------------------------------------------------------------------------------------
 // Persistent form of the direct-to-LDS kernel: one workgroup per CU walks the tile list
 // (linear tile id = blockIdx.x + i*gridDim.x, same XCD-grouped order as above) and the
 // k-tile pipeline runs straight through tile boundaries: while the last two k-tiles of a
@@ -972,6 +1202,45 @@ int tiled16_persist_launch(const void *X, const int64_t *off, const void *W, con
     return OPMX_OK;
 }
 
+template <typename T, int BM, int BN>
+int tiled16_plr_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
+                       int64_t K, int64_t N, int epilogue, void *Y, hipStream_t s)
+{
+    constexpr int smem = 2 * (BM + BN) * ROWB;
+    const bool sw = epilogue == OPMX_EPILOGUE_SWIGLU;
+    const int64_t ncols = sw ? N / 2 : N;
+    const int ntiles_n = static_cast<int>(ceil_div(ncols, sw ? BN / 2 : BN));
+    const int ntiles_m = static_cast<int>(max_mtiles(R, E, BM));
+    const int gnx = pick_gnx(ntiles_n);
+    const int64_t nblocks = linear_ids(gnx, ntiles_m, ntiles_n);
+    dim3 grid(static_cast<unsigned>(nblocks));
+    dim3 block(256);
+    static bool attr_done[2] = {false, false};
+    if (sw) {
+        auto kern = gemm_tiled16_plr_kernel<T, BM, BN, true>;
+        if (!attr_done[1]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    smem) != hipSuccess)
+                return OPMX_ERR_LAUNCH;
+            attr_done[1] = true;
+        }
+        kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_n, gnx);
+    } else {
+        auto kern = gemm_tiled16_plr_kernel<T, BM, BN, false>;
+        if (!attr_done[0]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    smem) != hipSuccess)
+                return OPMX_ERR_LAUNCH;
+            attr_done[0] = true;
+        }
+        kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_n, gnx);
+    }
+    OPMX_LAUNCH_CHECK();
+    return OPMX_OK;
+}
+
 template <typename T>
 int tiled16_impl(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
                  int64_t N, int epilogue, int variant, void *Y, hipStream_t s)
@@ -981,6 +1250,7 @@ int tiled16_impl(const void *X, const int64_t *off, const void *W, const void *B
         case 2: return tiled16_launch<T, 128, 128, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
         case 3: return tiled16_dlds_launch<T, 256, 256, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
         case 4: return tiled16_dlds_launch<T, 256, 256, 2, 4>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        case 7: return tiled16_plr_launch<T, 256, 256>(X, off, W, B, E, R, K, N, epilogue, Y, s);
         // the persistent kernels pipeline across tiles and need at least two k-tiles
         case 5:
             if (K < 2 * BK) return tiled16_dlds_launch<T, 256, 256, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
