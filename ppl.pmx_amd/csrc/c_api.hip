@@ -81,15 +81,10 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
         return launch_gemm_stream(X, off, W, B, E, R, K, N, dtype, epilogue, hint,
                                   env_int("OPMX_MOE_GEMM_STREAM_VARIANT", 0), Y, s);
     if (choice == 2) {
-        // 256x256 tiles (4 waves, 16x16x32 MFMA, direct-to-LDS) from 128 mean rows per expert on,
-        // else 128x128 (measured).
-        const int dflt = R / E >= 128 ? 14 : 0;
-        const int variant = env_int("OPMX_MOE_GEMM_TILED_VARIANT", dflt);
-        if (variant >= 7)   // 16x16x32 MFMA kernels, see tiled16_impl
-            return launch_gemm_tiled16(X, off, W, B, E, R, K, N, dtype, epilogue, variant - 7, Y, s);
-        if (variant == 6)   // 256x256 tiles fed by direct-to-LDS loads
-            return launch_gemm_tiled_dlds(X, off, W, B, E, R, K, N, dtype, epilogue, Y, s);
-        return launch_gemm_tiled(X, off, W, B, E, R, K, N, dtype, epilogue, variant, Y, s);
+        // 256x256 direct-to-LDS tiles from 128 mean rows per expert on, else 128x128 (measured).
+        const int dflt = R / E >= 128 ? 0 : 2;
+        return launch_gemm_tiled(X, off, W, B, E, R, K, N, dtype, epilogue,
+                                 env_int("OPMX_MOE_GEMM_TILED_VARIANT", dflt), Y, s);
     }
     return launch_gemm_generic(X, off, W, B, E, R, K, N, dtype, epilogue, Y, s);
 }

@@ -48,6 +48,13 @@ __device__ __forceinline__ float wave_sum(float v)
 
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
 
+// Hardware exp2 / reciprocal (about 1 ulp each in fp32): for epilogues whose result is rounded
+// to 16 bits anyway, where the accurate routine costs MFMA-idle time on every output tile.
+__device__ __forceinline__ float sigmoid_fast_(float x)
+{
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.44269504088896341f));
+}
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }

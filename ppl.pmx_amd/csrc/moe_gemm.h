@@ -126,12 +126,10 @@ __device__ __forceinline__ void zero_unowned_rows(T *__restrict__ Y, int64_t R, 
 
 int launch_gemm_generic(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
                         int64_t K, int64_t N, int dtype, int epilogue, void *Y, hipStream_t s);
+// variant: 0 = 256x256 direct-to-LDS kernel, 1 = 256x256 register-staged (8 waves),
+// 2 = 128x128 register-staged (4 waves).  off == nullptr: dense GEMM (one expert owns [0, R)).
 int launch_gemm_tiled(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
                       int64_t K, int64_t N, int dtype, int epilogue, int variant, void *Y, hipStream_t s);
-int launch_gemm_tiled16(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
-                        int64_t K, int64_t N, int dtype, int epilogue, int variant, void *Y, hipStream_t s);
-int launch_gemm_tiled_dlds(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
-                           int64_t K, int64_t N, int dtype, int epilogue, void *Y, hipStream_t s);
 int launch_gemm_stream(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
                        int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint, int variant, void *Y,
                        hipStream_t s);

@@ -187,7 +187,7 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
             if (SG) {                          // SwiGLU.py:15-16 on the fp32 accumulators, beta = 1
                 float u = acc[NG - 1][m][i];
                 if (Bias) u += to_f32(Bias[static_cast<int64_t>(mt.e) * N + ND + n]);
-                v = u * v * sigmoidf_(v);
+                v = u * v * sigmoid_fast_(v);
             }
             yrow[n] = from_f32<T>(v);
         }

@@ -2,17 +2,22 @@
 //
 //   Y[r, :] = X[r, :] W[e]^T (+ B[e])   for off[e] <= r < off[e+1]
 //
-// X [R,K] and W[e] [N,K] are both K-contiguous, so A and B fragments of
-// v_mfma_f32_32x32x16_{f16,bf16} are 16-byte loads.  A block owns a BM x BN
-// output tile of ONE expert (tiles never straddle experts; the tile list is
-// derived on the device from expert_offset, no host sync), stages X and W
-// tiles of BK=64 through XOR-swizzled LDS (two LDS buffers, one barrier per
-// k-tile, loads and LDS stores software-pipelined between the MFMA groups; with
-// ILV the instruction order inside a group is pinned to MFMA / fragment read /
-// LDS store / global load round-robin so the matrix pipe never waits behind a
-// burst of memory instructions) and accumulates in fp32.  Optional SwiGLU
-// epilogue on the accumulators (gate rows i and up rows N/2+i of W are placed
-// in the same lane by the B-tile row order).
+// X [R,K] and W[e] [N,K] are both K-contiguous, so MFMA fragments are 16-byte LDS reads.
+// A workgroup owns a BM x BN output tile of ONE expert (tiles never straddle experts; the
+// tile list is derived on the device from expert_offset, no host sync), streams BK=64
+// k-tiles of X and W through XOR-swizzled LDS and accumulates in fp32 with
+// v_mfma_f32_16x16x32 (measured ~10% more flops at the same board power than 32x32x16 on
+// random operands: a quarter of the accumulator registers move per instruction).  W is the
+// A operand and X the B operand, so a lane holds four consecutive output COLUMNS of a row.
+// Optional SwiGLU epilogue on the accumulators (gate rows i and up rows N/2+i of W are
+// placed in the same lane by the W-tile row order).
+//
+// Two kernels share the tile order, LDS layout and epilogues:
+//   gemm_tiled_dlds_kernel  256x256 tile, 4 waves, operands loaded straight into LDS, the
+//                           fragments of a whole k-tile held in registers.  Default from 128
+//                           mean rows per expert on.
+//   gemm_tiled_kernel       operands staged through registers (global -> VGPR -> LDS), any
+//                           BM x BN / wave layout; 128x128 tiles are the default below that.
 // Semantics: torch_function/MoeColumnParallelLinear.py:61-67,
 // torch_function/MoeRowParallelLinear.py:47-53, torch_function/SwiGLU.py:15-16.
 #include <cstdlib>
@@ -26,26 +31,251 @@ constexpr int BK = 64;                 // k elements per LDS tile (128 bytes per
 constexpr int ROWB = BK * 2;           // bytes per LDS row
 constexpr int CH = ROWB / 16;          // 16-byte chunks per row (8)
 
-// Byte offset of 16-byte chunk `chunk` of tile row `row`.  Rows are 128 bytes; the
-// XOR with (row>>1)&7 spreads 16 consecutive rows of one chunk column over all
-// sixteen 16-byte bank groups of a 256-byte LDS line pair (conflict-free b128 reads).
+// Byte offset of 16-byte chunk `chunk` of tile row `row`: 16 consecutive rows of one chunk
+// column land in sixteen different 16-byte bank groups (conflict-free b128 fragment reads).
 __device__ __forceinline__ int lds_off(int row, int chunk) { return row * ROWB + ((chunk ^ ((row >> 1) & 7)) << 4); }
 
-template <typename T, int BM, int BN, int WM, int WN, bool SWIGLU, bool ILV>
+// Clamped copy of expert_offset in LDS (values forced into a non-decreasing sequence inside
+// [0, R] when read, so a corrupt offset can never send a store outside Y).  Nothing to do for a
+// dense GEMM (off == nullptr).  Every thread must call it: it contains a block barrier.
+__device__ __forceinline__ void stage_offsets(const int64_t *__restrict__ off, int E, int64_t R, int64_t *s_off)
+{
+    if (off == nullptr) return;
+    for (int i = threadIdx.x; i <= E; i += blockDim.x) {
+        const int64_t v = off[i];
+        s_off[i] = v < 0 ? 0 : (v > R ? R : v);
+    }
+    __syncthreads();
+}
+
+// Number of row tiles of height BM over all experts: sum of ceil(rows_e / BM).
+__device__ __forceinline__ int count_mtiles(bool grouped, const int64_t *s_off, int E, int64_t R, int BM)
+{
+    if (!grouped) return static_cast<int>((R + BM - 1) / BM);
+    int64_t total = 0, prev = s_off[0];
+    for (int e = 0; e < E; ++e) {
+        int64_t hi = s_off[e + 1];
+        if (hi < prev) hi = prev;
+        total += (hi - prev + BM - 1) / BM;
+        prev = hi;
+    }
+    return __builtin_amdgcn_readfirstlane(static_cast<int>(total));
+}
+
+// Linear tile id -> (row tile, column tile); mtiles is the actual number of row tiles.
+// Workgroups are handed to the 8 XCDs round-robin by linear id and each XCD has its own L2, so
+// 256 consecutive ids ("a round", 32 per XCD) form a block of tiles in which every XCD owns a
+// compact sub-block: its 32 resident workgroups then share X- and W-tiles in that XCD's L2.
+//   gnx = 1, 2: XCDs side by side along n, each (32/gnx) x gnx tiles;
+//   gnx = 4   : rounds of 16 x 16 tiles, XCDs as 2 (m) x 4 (n), each 8 x 4 tiles (a third less
+//               L2 fill traffic than 16 x 2).  The last mtiles % 16 row tiles would leave XCDs
+//               idle in that layout; they are dealt out differently: XCD j takes the column
+//               tiles [j*ntiles_n/8, (j+1)*ntiles_n/8), walking m fastest.  ntiles_n % 16 == 0.
+//   gnx = 0   : plain row-major order, n fastest.
+// Ids that name no tile come back with tile_m >= mtiles.
+__device__ __forceinline__ void map_tile(int lin, int gnx, int mtiles, int ntiles_n, int &tile_m, int &tile_n)
+{
+    const int xcd = lin & 7, sl = (lin >> 3) & 31, round = lin >> 8;
+    if (gnx == 4) {
+        const int cols16 = ntiles_n / 16, full = mtiles / 16, rem = mtiles % 16;
+        const int ids_full = full * cols16 * 256;
+        if (lin < ids_full) {
+            tile_m = (round / cols16) * 16 + (xcd >> 2) * 8 + (sl & 7);
+            tile_n = (round % cols16) * 16 + (xcd & 3) * 4 + (sl >> 3);
+        } else {
+            const int s = (lin - ids_full) >> 3, cols = ntiles_n / 8;
+            if (rem > 0 && s < rem * cols) {
+                tile_m = full * 16 + s % rem;
+                tile_n = xcd * cols + s / rem;
+            } else {
+                tile_m = mtiles;
+                tile_n = 0;
+            }
+        }
+    } else if (gnx > 0) {
+        const int gm = 32 / gnx;
+        const int rounds_n = (ntiles_n + 8 * gnx - 1) / (8 * gnx);
+        tile_m = (round / rounds_n) * gm + sl % gm;
+        tile_n = (round % rounds_n) * (8 * gnx) + xcd * gnx + sl / gm;
+    } else {
+        tile_m = lin / ntiles_n;
+        tile_n = lin % ntiles_n;
+    }
+}
+
+// Linear tile id -> (row tile of one expert, column tile).  mt.rows == 0 when the id names no
+// work.  s_off: see stage_offsets (unused when `grouped` is false: one expert owns [0, R)).
+__device__ __forceinline__ void locate_tile(int lin, int gnx, int mtiles, int ntiles_n, bool grouped,
+                                            const int64_t *s_off, int E, int64_t R, int BM, MTile &mt, int &tile_n)
+{
+    int tile_m;
+    map_tile(lin, gnx, mtiles, ntiles_n, tile_m, tile_n);
+    mt.e = 0;
+    mt.rows = 0;
+    mt.row0 = 0;
+    if (tile_m >= mtiles || tile_n >= ntiles_n) return;
+    if (!grouped) {
+        mt.row0 = static_cast<int64_t>(tile_m) * BM;
+        const int64_t left = R - mt.row0;
+        mt.rows = left <= 0 ? 0 : static_cast<int>(left < BM ? left : BM);
+        return;
+    }
+    int64_t tile = tile_m, prev = s_off[0];
+    for (int e = 0; e < E; ++e) {
+        int64_t hi = s_off[e + 1];
+        if (hi < prev) hi = prev;
+        const int64_t nt = (hi - prev + BM - 1) / BM;
+        if (tile < nt) {
+            // block-uniform by construction; say so to the compiler (scalar registers)
+            const int64_t row0 = prev + tile * BM, left = hi - row0;
+            mt.e = __builtin_amdgcn_readfirstlane(e);
+            mt.row0 = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0 >> 32))) << 32) |
+                      static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0)));
+            mt.rows = __builtin_amdgcn_readfirstlane(static_cast<int>(left < BM ? left : BM));
+            return;
+        }
+        tile -= nt;
+        prev = hi;
+    }
+}
+
+// Host side of map_tile: the order to use and the number of linear ids it spans.
+inline int pick_gnx(int ntiles_n)
+{
+    // XCD-grouped orders only when the n-tiles split evenly over the rounds (else XCDs idle)
+    int gnx = ntiles_n % 16 == 0 ? 4 : (ntiles_n % 8 == 0 ? 1 : 0);
+    if (const char *v = std::getenv("OPMX_MOE_GEMM_GNX")) gnx = std::atoi(v);   // tuning knob
+    if (gnx != 0 && gnx != 1 && gnx != 2 && gnx != 4) gnx = 0;
+    if (gnx == 4 && ntiles_n % 16 != 0) gnx = 0;
+    return gnx;
+}
+inline int64_t linear_ids(int gnx, int ntiles_m, int ntiles_n)
+{
+    if (gnx == 4) return ceil_div(ntiles_n, 16) * ceil_div(ntiles_m, 16) * 256;
+    if (gnx > 0) return ceil_div(ntiles_n, 8 * gnx) * ceil_div(ntiles_m, 32 / gnx) * 256;
+    return static_cast<int64_t>(ntiles_n) * ntiles_m;
+}
+
+// Writes a wave's accumulators.  acc[j][i][v] is output row (X row) i*16 + lane%16 and output
+// column j*16 + (lane/16)*4 + v of the WTM x WTN wave tile: four consecutive columns per lane,
+// stored as one 8-byte word.  With SWIGLU sub-tiles j and j + TNS/2 hold gate and up columns.
+template <typename T, int WTM, int WTN, bool SWIGLU>
+__device__ __forceinline__ void tile_epilogue(float4_t (&acc)[WTN / 16][WTM / 16], const T *__restrict__ Bias,
+                                              T *__restrict__ Y, const MTile &mt, int64_t N, int64_t ncols,
+                                              int64_t n0, int wm, int wn, int lane)
+{
+    constexpr int TMS = WTM / 16, TNS = WTN / 16;
+    const int lrow = lane & 15, lk = lane >> 4;
+    const T *be = Bias ? Bias + static_cast<int64_t>(mt.e) * N : nullptr;
+    const bool vec_ok = (ncols % 4 == 0) && (reinterpret_cast<uintptr_t>(Y) % 8 == 0);
+#pragma unroll
+    for (int i = 0; i < TMS; ++i) {
+        const int row = wm * WTM + i * 16 + lrow;
+        if (row >= mt.rows) continue;
+        T *yrow = Y + (mt.row0 + row) * ncols;
+#pragma unroll
+        for (int j = 0; j < (SWIGLU ? TNS / 2 : TNS); ++j) {
+            const int64_t n = (SWIGLU ? n0 + wn * (WTN / 2) : n0 + wn * WTN) + j * 16 + lk * 4;
+            if (n >= ncols) continue;
+            float val[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int64_t nn = n + v < ncols ? n + v : ncols - 1;
+                float g = acc[j][i][v] + (be ? to_f32(be[nn]) : 0.0f);
+                if (SWIGLU) {
+                    const float up = acc[j + TNS / 2][i][v] + (be ? to_f32(be[ncols + nn]) : 0.0f);
+                    g = up * g * sigmoid_fast_(g);
+                }
+                val[v] = g;
+            }
+            if (vec_ok && n + 3 < ncols) {
+                T out[4];
+#pragma unroll
+                for (int v = 0; v < 4; ++v) out[v] = from_f32<T>(val[v]);
+                *reinterpret_cast<uint2 *>(yrow + n) = *reinterpret_cast<const uint2 *>(out);
+            } else {
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (n + v < ncols) yrow[n + v] = from_f32<T>(val[v]);
+            }
+        }
+    }
+}
+
+// Same result as tile_epilogue, but staged through a wave-private LDS region (WTM rows of the
+// wave's output columns, 16-byte chunks XOR-swizzled by row) so that global memory sees whole
+// rows of the wave tile: each store instruction writes 1 KiB as runs of 128/256 contiguous
+// bytes instead of 32-byte pieces.  No block barrier is needed (a wave only touches its own
+// region, and its LDS operations execute in order); the caller guarantees that no wave still
+// reads operand tiles from LDS.  Requires ncols % 8 == 0 and a 16-byte aligned Y.
+template <typename T, int WTM, int WTN, bool SWIGLU>
+__device__ __forceinline__ void tile_epilogue_lds(float4_t (&acc)[WTN / 16][WTM / 16], const T *__restrict__ Bias,
+                                                  T *__restrict__ Y, const MTile &mt, int64_t N, int64_t ncols,
+                                                  int64_t n0, int wm, int wn, int lane, char *wave_lds)
+{
+    constexpr int TMS = WTM / 16, TNS = WTN / 16, NO = SWIGLU ? TNS / 2 : TNS;
+    constexpr int ROWP = NO * 16 * 2;          // bytes per staged row
+    constexpr int CH16 = ROWP / 16;            // 16-byte chunks per staged row
+    constexpr int RPI = 1024 / ROWP;           // rows per wave-wide 16-byte access
+    const int lrow = lane & 15, lk = lane >> 4;
+    const T *be = Bias ? Bias + static_cast<int64_t>(mt.e) * N : nullptr;
+    const int64_t nw0 = (SWIGLU ? n0 + wn * (WTN / 2) : n0 + wn * WTN);   // first output column of this wave
+#pragma unroll
+    for (int i = 0; i < TMS; ++i) {
+        const int row = i * 16 + lrow;
+#pragma unroll
+        for (int j = 0; j < NO; ++j) {
+            const int64_t n = nw0 + j * 16 + lk * 4;
+            T out[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int64_t nn = n + v < ncols ? n + v : ncols - 1;
+                float g = acc[j][i][v] + (be ? to_f32(be[nn]) : 0.0f);
+                if (SWIGLU) {
+                    const float up = acc[j + TNS / 2][i][v] + (be ? to_f32(be[ncols + nn]) : 0.0f);
+                    g = up * g * sigmoid_fast_(g);
+                }
+                out[v] = from_f32<T>(g);
+            }
+            const int chunk = j * 2 + (lk >> 1);
+            *reinterpret_cast<uint2 *>(wave_lds + row * ROWP + ((chunk ^ (row % CH16)) << 4) + (lk & 1) * 8) =
+                *reinterpret_cast<const uint2 *>(out);
+        }
+    }
+#pragma unroll
+    for (int rr = 0; rr < WTM / RPI; ++rr) {
+        const int row = rr * RPI + lane / CH16, c = lane % CH16;
+        const u32x4 v = *reinterpret_cast<const u32x4 *>(wave_lds + row * ROWP + ((c ^ (row % CH16)) << 4));
+        const int grow = wm * WTM + row;
+        const int64_t n = nw0 + c * 8;
+        if (grow < mt.rows && n < ncols)       // ncols % 8 == 0: a chunk is inside or outside as a whole
+            *reinterpret_cast<u32x4 *>(Y + (mt.row0 + grow) * ncols + n) = v;
+    }
+}
+
+// Register-staged kernel: two LDS buffers, ONE register set staging global -> LDS, one barrier
+// per k-tile.  A k-tile is four MFMA groups (K32 step 0/1 x lower/upper half of the wave's X
+// rows); each group prefetches the fragments of the next one and carries its share of the
+// LDS stores / global loads, the order inside a group pinned with sched_group_barrier.
+template <typename T, int BM, int BN, int WM, int WN, bool SWIGLU>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__restrict__ X,
                                                                   const int64_t *__restrict__ off,
                                                                   const T *__restrict__ W,
                                                                   const T *__restrict__ Bias, int E, int64_t R,
                                                                   int64_t K, int64_t N, T *__restrict__ Y,
-                                                                  int ntiles_m, int ntiles_n, int gnx)
+                                                                  int ntiles_n, int gnx)
 {
     constexpr int NT = WM * WN * 64;
-    constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
+    constexpr int WTM = BM / WM, WTN = BN / WN;          // wave tile: WTM X-rows x WTN W-rows
+    constexpr int TMS = WTM / 16, TNS = WTN / 16;        // 16x16 sub-tiles per wave
+    constexpr int HM = TMS / 2;                          // X sub-tiles per MFMA group
     constexpr int BNO = SWIGLU ? BN / 2 : BN;            // output columns per tile
     constexpr int LA = BM * CH / NT, LB = BN * CH / NT;  // 16-byte loads per thread per k-tile
+    constexpr int RSTEP = NT / CH;                       // tile rows between a thread's consecutive loads
     constexpr int STAGE = (BM + BN) * ROWB;
     static_assert(BM * CH % NT == 0 && BN * CH % NT == 0, "tile/threads mismatch");
-    static_assert(!SWIGLU || TN % 2 == 0, "SwiGLU needs an even number of n sub-tiles per wave");
+    static_assert(TMS % 2 == 0 && RSTEP % 16 == 0, "wave tile too small");
+    static_assert(!SWIGLU || TNS % 2 == 0, "SwiGLU needs an even number of n sub-tiles per wave");
     using frag = typename Mfma<T>::frag;
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -54,24 +284,11 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
     const int64_t ncols = SWIGLU ? N / 2 : N;
     zero_unowned_rows(Y, R, ncols, off, E);
 
-    // Block -> tile map.  Workgroups are handed to the 8 XCDs round-robin by linear id and
-    // each XCD has its own L2, so 256 consecutive ids ("a round": 32 per XCD) are laid out
-    // as a gm x (8*gnx) block of tiles in which XCD j owns a compact gm x gnx sub-block:
-    // its 32 resident blocks share gm X-tiles and gnx W-tiles in L2, and all 8 XCDs share
-    // the round's X-tiles through the memory-side cache.  Rounds walk n first, then m.
-    int tile_m, tile_n;
-    if (gnx > 0) {
-        const int gm = 32 / gnx;
-        const int lin = blockIdx.x, xcd = lin & 7, slot = (lin >> 3) & 31, round = lin >> 8;
-        const int rounds_n = (ntiles_n + 8 * gnx - 1) / (8 * gnx);
-        tile_m = (round / rounds_n) * gm + slot % gm;
-        tile_n = (round % rounds_n) * (8 * gnx) + xcd * gnx + slot / gm;
-    } else {                       // plain row-major order, n fastest
-        tile_m = blockIdx.x / ntiles_n;
-        tile_n = blockIdx.x % ntiles_n;
-    }
-    if (tile_m >= ntiles_m || tile_n >= ntiles_n) return;
-    const MTile mt = find_mtile(off, E, R, BM, tile_m, s_off);
+    stage_offsets(off, E, R, s_off);
+    MTile mt;
+    int tile_n;
+    locate_tile(blockIdx.x, gnx, count_mtiles(off != nullptr, s_off, E, R, BM), ntiles_n, off != nullptr, s_off, E, R,
+                BM, mt, tile_n);
     if (mt.rows == 0) return;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -80,20 +297,23 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
     const T *Xt = X + mt.row0 * K;
     const T *We = W + static_cast<int64_t>(mt.e) * N * K;
 
-    // per-thread global offsets (elements) and LDS offsets (bytes) of its loads
-    int a_src[LA], a_dst[LA], b_src[LB], b_dst[LB];
+    // Staging: load q of a thread covers tile row tid/8 + RSTEP*q, 16-byte chunk tid%8.
+    // RSTEP is a multiple of 16, so the swizzle term is the same for all of them and the
+    // LDS destinations differ by compile-time constants.
+    uint32_t a_src[LA], b_src[LB];   // byte offsets from the (uniform) tile base: scalar base + 32-bit lane offset loads
+    const int srow = tid / CH, sc = tid % CH;
+    const int dst0 = lds_off(srow, sc);
 #pragma unroll
     for (int i = 0; i < LA; ++i) {
-        const int q = tid + NT * i, row = q / CH, c = q % CH;
+        const int row = srow + RSTEP * i;
         const int r = row < mt.rows ? row : mt.rows - 1;
-        a_src[i] = static_cast<int>(r * K + c * 8);
-        a_dst[i] = lds_off(row, c);
+        a_src[i] = static_cast<uint32_t>((r * K + sc * 8) * 2);
     }
 #pragma unroll
     for (int i = 0; i < LB; ++i) {
-        const int q = tid + NT * i, row = q / CH, c = q % CH;
+        const int row = srow + RSTEP * i;
         int64_t wrow;
-        if (SWIGLU) {
+        if (SWIGLU) {      // wave w's rows: WTN/2 gate rows, then the WTN/2 matching up rows
             const int w = row / WTN, jj = row % WTN, half = jj / (WTN / 2);
             int64_t ii = n0 + w * (WTN / 2) + jj % (WTN / 2);
             ii = ii < ncols ? ii : ncols - 1;
@@ -101,75 +321,91 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
         } else {
             wrow = n0 + row < N ? n0 + row : N - 1;
         }
-        b_src[i] = static_cast<int>(wrow * K + c * 8);
-        b_dst[i] = BM * ROWB + lds_off(row, c);
+        b_src[i] = static_cast<uint32_t>((wrow * K + sc * 8) * 2);
     }
 
-    float16_t acc[TM][TN];
+    float4_t acc[TNS][TMS];
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int j = 0; j < TNS; ++j)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+        for (int i = 0; i < TMS; ++i)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+            for (int v = 0; v < 4; ++v) acc[j][i][v] = 0.0f;
 
-    // Software pipeline over k-tiles: ONE register set for global->LDS staging, two LDS
-    // buffers, double-buffered MFMA fragments, one barrier per k-tile.
-    // An iteration (tile kt in LDS buffer kt&1) has KS = BK/16 MFMA groups.  Group g
-    //   - prefetches the fragments of group g+1 into the other fragment set,
-    //   - issues its MFMAs on fragments that were fetched one group earlier,
-    //   - (g < KS-1) stores its share of the staging registers (tile kt+1, loaded one
-    //     iteration ago) into LDS buffer (kt+1)&1 and reloads them with tile kt+2.
-    // The barrier sits BEFORE the last group: by then every wave has finished reading
-    // buffer kt&1 (the last group's fragments are already in registers) and writing
-    // buffer (kt+1)&1, so the last group prefetches the first fragments of tile kt+1
-    // while its MFMAs run, and the next iteration may overwrite buffer kt&1.
-    constexpr int KS = BK / 16, NQ = LA + LB, QPK = (NQ + KS - 2) / (KS - 1);
-    // first MFMA slot that carries an LDS-store/global-load pair: LDS stores stay behind the group's fragment reads
-    constexpr int ILV0 = TM + TN < TM * TN - QPK ? TM + TN : (TM * TN - QPK > 0 ? TM * TN - QPK : 0);
+    // Pipeline over k-tiles (tile kt sits in LDS buffer kt&1).  Group g = 2*s + h of a
+    // k-tile multiplies the K32 step s of the W fragments wf[s] with X fragments xf[h]
+    // (half h of the wave's X sub-tiles), after prefetching the fragments of group g+1:
+    //   g+1 odd : xf[1] <- upper X half of the same step
+    //   g+1 even: xf[0] <- lower X half and wf[s^1] <- W fragments of the next step.
+    // Groups 0..2 also store their share of the staging registers (tile kt+1, loaded one
+    // iteration ago) into buffer (kt+1)&1 and reload them with tile kt+2.  The barrier sits
+    // before group 3, whose prefetch already reads tile kt+1.
+    constexpr int KS = 4, NQ = LA + LB, QPK = (NQ + KS - 2) / (KS - 1), NM = HM * TNS;
     u32x4 rq[NQ];
-    frag fa[2][TM], fb[2][TN];
+    frag xf[2][HM], wf[2][TNS];
     const int nk = static_cast<int>(K / BK);
-    const int lrow = lane & 31, lk = lane >> 5;
-    int fa_off[TM], fb_off[TN];      // LDS offsets of this lane's fragments for chunk pair 0
-#pragma unroll
-    for (int i = 0; i < TM; ++i) fa_off[i] = (wm * WTM + i * 32 + lrow) * ROWB;
-#pragma unroll
-    for (int j = 0; j < TN; ++j) fb_off[j] = BM * ROWB + (wn * WTN + j * 32 + lrow) * ROWB;
-    const int swz = (lrow >> 1) & 7;  // (row>>1)&7 of every fragment row of this lane (rows differ by multiples of 32)
+    const int lrow = lane & 15, lk = lane >> 4;
+    const int swz = (lrow >> 1) & 7;                 // fragment rows differ from lrow by multiples of 16
+    const int x_off = (wm * WTM + lrow) * ROWB;
+    const int w_off = BM * ROWB + (wn * WTN + lrow) * ROWB;
+    const int co0 = ((lk ^ swz) << 4), co1 = (((4 + lk) ^ swz) << 4);
 
 #define OPMX_LOADQ(Q, KT)                                                                          \
     do {                                                                                           \
         const int64_t ko_ = static_cast<int64_t>(KT) * BK;                                         \
-        if ((Q) < LA) rq[Q] = *reinterpret_cast<const u32x4 *>(Xt + a_src[(Q) < LA ? (Q) : 0] + ko_); \
-        else rq[Q] = *reinterpret_cast<const u32x4 *>(We + b_src[(Q) < LA ? 0 : (Q)-LA] + ko_);    \
+        if ((Q) < LA)                                                                              \
+            rq[Q] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(Xt + ko_) +    \
+                                                     a_src[(Q) < LA ? (Q) : 0]);                   \
+        else                                                                                       \
+            rq[Q] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(We + ko_) +    \
+                                                     b_src[(Q) < LA ? 0 : (Q)-LA]);                \
     } while (0)
 #define OPMX_DRAINQ(Q, BUF)                                                                        \
     do {                                                                                           \
-        char *dst_ = smem + (BUF)*STAGE;                                                           \
-        if ((Q) < LA) *reinterpret_cast<u32x4 *>(dst_ + a_dst[(Q) < LA ? (Q) : 0]) = rq[Q];        \
-        else *reinterpret_cast<u32x4 *>(dst_ + b_dst[(Q) < LA ? 0 : (Q)-LA]) = rq[Q];              \
+        char *dst_ = smem + (BUF)*STAGE + dst0;                                                    \
+        if ((Q) < LA) *reinterpret_cast<u32x4 *>(dst_ + (Q)*RSTEP * ROWB) = rq[Q];                 \
+        else *reinterpret_cast<u32x4 *>(dst_ + BM * ROWB + ((Q)-LA) * RSTEP * ROWB) = rq[Q];       \
     } while (0)
-#define OPMX_FRAGS(SET, BUF, G)                                                                    \
+    // fragments of group G of the tile in buffer BUF
+#define OPMX_FRAGS(BUF, G)                                                                         \
     do {                                                                                           \
-        const char *src_ = smem + (BUF)*STAGE;                                                     \
-        const int co_ = ((((G)*2 + lk) ^ swz) << 4);                                               \
-        _Pragma("unroll") for (int i = 0; i < TM; ++i)                                             \
-            fa[SET][i] = *reinterpret_cast<const frag *>(src_ + fa_off[i] + co_);                  \
-        _Pragma("unroll") for (int j = 0; j < TN; ++j)                                             \
-            fb[SET][j] = *reinterpret_cast<const frag *>(src_ + fb_off[j] + co_);                  \
+        const char *src_ = smem + (BUF)*STAGE + (((G) >> 1) ? co1 : co0);                          \
+        if (((G)&1) == 0) {                                                                        \
+            _Pragma("unroll") for (int i = 0; i < HM; ++i)                                         \
+                xf[0][i] = *reinterpret_cast<const frag *>(src_ + x_off + i * 16 * ROWB);          \
+            _Pragma("unroll") for (int j = 0; j < TNS; ++j)                                        \
+                wf[((G) >> 1) & 1][j] = *reinterpret_cast<const frag *>(src_ + w_off + j * 16 * ROWB); \
+        } else {                                                                                   \
+            _Pragma("unroll") for (int i = 0; i < HM; ++i)                                         \
+                xf[1][i] = *reinterpret_cast<const frag *>(src_ + x_off + (HM + i) * 16 * ROWB);   \
+        }                                                                                          \
     } while (0)
-#define OPMX_MMA(SET)                                                                              \
+#define OPMX_MMA(G)                                                                                \
     do {                                                                                           \
-        _Pragma("unroll") for (int i = 0; i < TM; ++i)                                             \
-            _Pragma("unroll") for (int j = 0; j < TN; ++j)                                         \
-                acc[i][j] = Mfma<T>::m32(fa[SET][i], fb[SET][j], acc[i][j]);                       \
+        _Pragma("unroll") for (int i = 0; i < HM; ++i)                                             \
+            _Pragma("unroll") for (int j = 0; j < TNS; ++j)                                        \
+                acc[j][((G)&1) * HM + i] =                                                         \
+                    Mfma<T>::m16(wf[((G) >> 1) & 1][j], xf[(G)&1][i], acc[j][((G)&1) * HM + i]);   \
+    } while (0)
+    // Pin the order inside a group: one fragment read behind each of the first MFMAs, then
+    // one LDS-store / global-load pair behind each of the following ones.
+#define OPMX_ORDER(NREAD, NPAIR, DRAIN, LOAD)                                                      \
+    do {                                                                                           \
+        _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                     \
+            if (m < (NREAD)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                    \
+            const int p0 = (NREAD) < NM - (NPAIR) ? (NREAD) : (NM - (NPAIR) > 0 ? NM - (NPAIR) : 0); \
+            if (m >= p0 && m < p0 + (NPAIR)) {                                                     \
+                if (DRAIN) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                      \
+                if (LOAD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                       \
+            }                                                                                      \
+        }                                                                                          \
     } while (0)
 #define OPMX_ITER(KT, DRAIN, LOAD, NEXT)                                                           \
     do {                                                                                           \
         _Pragma("unroll") for (int g = 0; g < KS - 1; ++g) {                                       \
-            OPMX_FRAGS((g + 1) & 1, (KT)&1, g + 1);                                                \
-            OPMX_MMA(g & 1);                                                                       \
+            OPMX_FRAGS((KT)&1, g + 1);                                                             \
+            OPMX_MMA(g);                                                                           \
             _Pragma("unroll") for (int qq = 0; qq < QPK; ++qq) {                                   \
                 const int q = g * QPK + qq;                                                        \
                 if (q < NQ) {                                                                      \
@@ -177,27 +413,14 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
                     if (LOAD) OPMX_LOADQ(q, (KT) + 2);                                             \
                 }                                                                                  \
             }                                                                                      \
-            if (ILV) {                                                                             \
-                _Pragma("unroll") for (int m = 0; m < TM * TN; ++m) {                              \
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                             \
-                    if (m < TM + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);            \
-                    if (m >= ILV0 && m < ILV0 + QPK && g * QPK + (m - ILV0) < NQ) {                \
-                        if (DRAIN) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);              \
-                        if (LOAD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);               \
-                    }                                                                              \
-                }                                                                                  \
-            }                                                                                      \
+            OPMX_ORDER(((g + 1) & 1) ? HM : HM + TNS,                                              \
+                       (NQ - g * QPK < QPK ? (NQ - g * QPK > 0 ? NQ - g * QPK : 0) : QPK), DRAIN, LOAD); \
             __builtin_amdgcn_sched_barrier(0);                                                     \
         }                                                                                          \
         __syncthreads();                                                                           \
-        if (NEXT) OPMX_FRAGS(KS & 1, ((KT) + 1) & 1, 0);                                           \
-        OPMX_MMA((KS - 1) & 1);                                                                    \
-        if (ILV && (NEXT)) {                                                                       \
-            _Pragma("unroll") for (int m = 0; m < TM * TN; ++m) {                                  \
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                 \
-                if (m < TM + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                \
-            }                                                                                      \
-        }                                                                                          \
+        if (NEXT) OPMX_FRAGS(((KT) + 1) & 1, 0);                                                   \
+        OPMX_MMA(KS - 1);                                                                          \
+        if (NEXT) OPMX_ORDER(HM + TNS, 0, false, false);                                           \
         __builtin_amdgcn_sched_barrier(0);                                                         \
     } while (0)
 
@@ -210,9 +433,8 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
         for (int q = 0; q < NQ; ++q) OPMX_LOADQ(q, 1);
     }
     __syncthreads();
-    OPMX_FRAGS(0, 0, 0);
+    OPMX_FRAGS(0, 0);
     {
-        static_assert(KS % 2 == 0, "fragment set parity must repeat every k-tile");
         int kt = 0;
         for (; kt + 2 < nk; ++kt) OPMX_ITER(kt, true, true, true);
         if (kt + 1 < nk) {
@@ -222,55 +444,243 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
         OPMX_ITER(kt, false, false, false);
     }
 #undef OPMX_ITER
+#undef OPMX_ORDER
 #undef OPMX_MMA
 #undef OPMX_FRAGS
 #undef OPMX_DRAINQ
 #undef OPMX_LOADQ
 
-    // epilogue: acc[i][j][v] is row (v/4)*8 + (lane/32)*4 + v%4, column lane%32 of its 32x32 sub-tile
-    const T *be = Bias ? Bias + static_cast<int64_t>(mt.e) * N : nullptr;
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < (SWIGLU ? TN / 2 : TN); ++j) {
-            const int64_t n = SWIGLU ? n0 + wn * (WTN / 2) + j * 32 + lrow : n0 + wn * WTN + j * 32 + lrow;
-            if (n >= ncols) continue;
-            const float bg = be ? to_f32(be[n]) : 0.0f;
-            const float bu = (SWIGLU && be) ? to_f32(be[ncols + n]) : 0.0f;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = wm * WTM + i * 32 + (v / 4) * 8 + lk * 4 + (v % 4);
-                if (row >= mt.rows) continue;
-                float val = acc[i][j][v] + bg;
-                if (SWIGLU) {
-                    const float up = acc[i][j + TN / 2][v] + bu;
-                    val = up * val * sigmoidf_(val);
-                }
-                Y[(mt.row0 + row) * ncols + n] = from_f32<T>(val);
-            }
-        }
+    // every wave passed the last barrier with its final fragments in registers: LDS is free
+    if (ncols % 8 == 0 && reinterpret_cast<uintptr_t>(Y) % 16 == 0)
+        tile_epilogue_lds<T, WTM, WTN, SWIGLU>(acc, Bias, Y, mt, N, ncols, n0, wm, wn, lane,
+                                               smem + wave * (WTM * (SWIGLU ? WTN / 2 : WTN) * 2));
+    else
+        tile_epilogue<T, WTM, WTN, SWIGLU>(acc, Bias, Y, mt, N, ncols, n0, wm, wn, lane);
 }
 
-template <typename T, int BM, int BN, int WM, int WN, bool ILV = false>
+// ---------------------------------------------------------------------------------------
+// Pieces of the direct-to-LDS kernel below.
+#define OPMX_LPTR(p) ((void __attribute__((address_space(3))) *)(p))
+
+// Block barrier WITHOUT a memory fence (a fence would wait for every in-flight direct-to-LDS
+// load).  The caller orders explicitly: s_waitcnt vmcnt(0) for the tile it publishes,
+// lgkmcnt(0) here for its own LDS reads of the buffer being retired.
+__device__ __forceinline__ void barrier_no_fence()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+// Raw buffer descriptor over [base, base + 4 GiB): loads through it take a scalar base, a
+// scalar offset and a 32-bit lane offset.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t raw_descriptor(const void *base)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, static_cast<int>(0xFFFFFFFFu), 0x00020000);
+}
+
+// 16 bytes per lane from descriptor + soff + voff straight into LDS at lds + 16*lane (lds is
+// wave-uniform).
+__device__ __forceinline__ void load_to_lds_16(__amdgpu_buffer_rsrc_t r, char *lds, uint32_t voff, int soff)
+{
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, OPMX_LPTR(lds), 16, voff, soff, 0, 0);
+}
+
+// ---------------------------------------------------------------------------------------
+// Direct-to-LDS, 4 waves, fragments of a whole k-tile held in registers.  Each wave reads all
+// 32 fragments of k-tile kt (128 VGPRs) by the first third of the k-tile, so the LDS buffer is
+// free again a good k-tile before it is needed and the loads of k-tile kt+2 get more than a
+// whole k-tile to land behind MFMAs: the slowest load of the slowest wave, which every wave
+// waits for at the barrier, stops being the pace setter.  Two barriers per k-tile:
+//   A (group 1, after this wave's last fragment read of buffer kt&1 returned): buffer free ->
+//     16 loads of k-tile kt+2 into it, one every third MFMA of groups 1-2;
+//   B (before group 3, after s_waitcnt vmcnt(16): this wave's loads of k-tile kt+1 landed) ->
+//     group 3 reads the first fragments of k-tile kt+1.
+// MFMAs are volatile asm (accumulators pinned to the 256 accumulation registers), so the
+// source order below is the issue order.
+template <typename T, int BM, int BN, bool SWIGLU>
+__global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restrict__ X,
+                                                               const int64_t *__restrict__ off,
+                                                               const T *__restrict__ W,
+                                                               const T *__restrict__ Bias, int E, int64_t R,
+                                                               int64_t K, int64_t N, T *__restrict__ Y,
+                                                               int ntiles_n, int gnx)
+{
+    constexpr int WM = 2, WN = 2, NW = 4;
+    constexpr int WTM = BM / WM, WTN = BN / WN, TMS = WTM / 16, TNS = WTN / 16, HM = TMS / 2;
+    constexpr int BNO = SWIGLU ? BN / 2 : BN;
+    constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW, NL = LA + LB;   // 1 KiB wave loads per k-tile
+    constexpr int STAGE = (BM + BN) * ROWB;
+    constexpr int NM = HM * TNS;
+    static_assert(HM == 4 && TNS == 8 && NL == 16, "the schedule below is written for 128x128 wave tiles");
+    using frag = typename Mfma<T>::frag;
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    __shared__ int64_t s_off[OPMX_MOE_MAX_EXPERTS + 1];
+
+    const int64_t ncols = SWIGLU ? N / 2 : N;
+    zero_unowned_rows(Y, R, ncols, off, E);
+    stage_offsets(off, E, R, s_off);
+    MTile mt;
+    int tile_n;
+    locate_tile(blockIdx.x, gnx, count_mtiles(off != nullptr, s_off, E, R, BM), ntiles_n, off != nullptr, s_off, E, R,
+                BM, mt, tile_n);
+    if (mt.rows == 0) return;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int64_t n0 = static_cast<int64_t>(tile_n) * BNO;
+    const __amdgpu_buffer_rsrc_t rx = raw_descriptor(X + mt.row0 * K);
+    const __amdgpu_buffer_rsrc_t rw = raw_descriptor(W + static_cast<int64_t>(mt.e) * N * K);
+
+    // this lane's share of the wave loads: tile row 8*(wave*L+i) + lane/8, LDS slot lane%8
+    const int lrow8 = lane >> 3, slot = lane & 7;
+    uint32_t a_src[LA], b_src[LB];     // byte offsets from the tile's X / W base at k = 0
+#pragma unroll
+    for (int i = 0; i < LA; ++i) {
+        const int row = (wave * LA + i) * 8 + lrow8;
+        const int r = row < mt.rows ? row : mt.rows - 1;
+        const int c = slot ^ ((row >> 1) & 7);
+        a_src[i] = static_cast<uint32_t>((r * K + c * 8) * 2);
+    }
+#pragma unroll
+    for (int i = 0; i < LB; ++i) {
+        const int row = (wave * LB + i) * 8 + lrow8;
+        int64_t wrow;
+        if (SWIGLU) {
+            const int w = row / WTN, jj = row % WTN, half = jj / (WTN / 2);
+            int64_t ii = n0 + w * (WTN / 2) + jj % (WTN / 2);
+            ii = ii < ncols ? ii : ncols - 1;
+            wrow = half * ncols + ii;
+        } else {
+            wrow = n0 + row < N ? n0 + row : N - 1;
+        }
+        const int c = slot ^ ((row >> 1) & 7);
+        b_src[i] = static_cast<uint32_t>((wrow * K + c * 8) * 2);
+    }
+    const int a_lds = wave * LA * 1024, b_lds = BM * ROWB + wave * LB * 1024;   // wave-uniform
+
+    float4_t acc[TNS][TMS];
+#pragma unroll
+    for (int j = 0; j < TNS; ++j)
+#pragma unroll
+        for (int i = 0; i < TMS; ++i)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[j][i][v] = 0.0f;
+
+    const int nk = static_cast<int>(K / BK);
+    const int lrow = lane & 15, lk = lane >> 4;
+    const int swz = (lrow >> 1) & 7;
+    const int x_off = (wm * WTM + lrow) * ROWB;
+    const int w_off = BM * ROWB + (wn * WTN + lrow) * ROWB;
+    const int co0 = ((lk ^ swz) << 4), co1 = (((4 + lk) ^ swz) << 4);
+    frag xf[2][2][HM], wf[2][TNS];      // [k32 step][X half][sub-tile], [k32 step][sub-tile]
+
+    // wave load Q of k-tile KT into buffer BUF: Q < LA -> X rows, else W rows
+#define OPMX_ISSUE1(KT, BUF, Q)                                                                    \
+    do {                                                                                           \
+        char *st_ = smem + (BUF)*STAGE;                                                            \
+        const int kb_ = (KT)*ROWB;                                                                 \
+        if ((Q) < LA) load_to_lds_16(rx, st_ + a_lds + (Q)*1024, a_src[(Q) < LA ? (Q) : 0], kb_);  \
+        else load_to_lds_16(rw, st_ + b_lds + ((Q)-LA) * 1024, b_src[(Q) < LA ? 0 : (Q)-LA], kb_); \
+    } while (0)
+#define OPMX_XFRAG(BUF, S, H, I)                                                                   \
+    xf[S][H][I] = *reinterpret_cast<const frag *>(smem + (BUF)*STAGE + ((S) ? co1 : co0) + x_off + ((H)*HM + (I)) * 16 * ROWB)
+#define OPMX_WFRAG(BUF, S, J)                                                                      \
+    wf[S][J] = *reinterpret_cast<const frag *>(smem + (BUF)*STAGE + ((S) ? co1 : co0) + w_off + (J)*16 * ROWB)
+#define OPMX_MF(S, H, m) Mfma<T>::m16_acc(wf[S][(m) % TNS], xf[S][H][(m) / TNS], acc[(m) % TNS][(H)*HM + (m) / TNS])
+    // k-tile in buffer B.  LD2: k-tile KT+2 exists (loaded into buffer B).  NEXT: k-tile KT+1 exists.
+#define OPMX_ITER(KT, B, LD2, NEXT)                                                                \
+    do {                                                                                           \
+        _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
+            OPMX_MF(0, 0, m);                                                                      \
+            if (m % 2 == 0) {                                                                      \
+                const int r = m / 2;                                                               \
+                if (r < 4) OPMX_XFRAG(B, 0, 1, r < 4 ? r : 0);                                     \
+                else if (r < 8) OPMX_XFRAG(B, 1, 0, (r >= 4 && r < 8) ? r - 4 : 0);                \
+                else OPMX_WFRAG(B, 1, r >= 8 ? r - 8 : 0);                                         \
+            }                                                                                      \
+        }                                                                                          \
+        _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
+            OPMX_MF(0, 1, m);                                                                      \
+            if (m < 4) OPMX_XFRAG(B, 1, 1, m < 4 ? m : 0);                                         \
+            if (m == 10) barrier_no_fence();                                                       \
+            if ((LD2) && m >= 11 && (m - 11) % 3 == 0) OPMX_ISSUE1((KT) + 2, B, (m - 11) / 3);     \
+        }                                                                                          \
+        _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
+            OPMX_MF(1, 0, m);                                                                      \
+            if ((LD2) && m % 3 == 0 && m / 3 < 9) OPMX_ISSUE1((KT) + 2, B, 7 + m / 3);             \
+        }                                                                                          \
+        if (LD2) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");                                 \
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                      \
+        __builtin_amdgcn_s_barrier();                                                              \
+        asm volatile("" ::: "memory");                                                             \
+        _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
+            OPMX_MF(1, 1, m);                                                                      \
+            if ((NEXT) && m < 4) OPMX_XFRAG((B) ^ 1, 0, 0, m < 4 ? m : 0);                         \
+            else if ((NEXT) && m < 12) OPMX_WFRAG((B) ^ 1, 0, (m >= 4 && m < 12) ? m - 4 : 0);     \
+        }                                                                                          \
+    } while (0)
+
+    // prologue: k-tile 0 -> buffer 0, k-tile 1 -> buffer 1, wait for k-tile 0
+#pragma unroll
+    for (int q = 0; q < NL; ++q) OPMX_ISSUE1(0, 0, q);
+    if (nk > 1) {
+#pragma unroll
+        for (int q = 0; q < NL; ++q) OPMX_ISSUE1(1, 1, q);
+        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < HM; ++i) OPMX_XFRAG(0, 0, 0, i);
+#pragma unroll
+    for (int j = 0; j < TNS; ++j) OPMX_WFRAG(0, 0, j);
+    {
+        int kt = 0, b = 0;
+        for (; kt + 2 < nk; ++kt, b ^= 1) OPMX_ITER(kt, b, true, true);
+        if (kt + 1 < nk) {
+            OPMX_ITER(kt, b, false, true);
+            ++kt;
+            b ^= 1;
+        }
+        OPMX_ITER(kt, b, false, false);
+    }
+#undef OPMX_ITER
+#undef OPMX_MF
+#undef OPMX_WFRAG
+#undef OPMX_XFRAG
+#undef OPMX_ISSUE1
+
+    // asm MFMAs are opaque to the compiler's hazard padding: let the last ones retire
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    // after the last barrier no wave reads operand tiles any more: LDS is free for the epilogue
+    if (ncols % 8 == 0 && reinterpret_cast<uintptr_t>(Y) % 16 == 0)
+        tile_epilogue_lds<T, WTM, WTN, SWIGLU>(acc, Bias, Y, mt, N, ncols, n0, wm, wn, lane,
+                                               smem + wave * (WTM * (SWIGLU ? WTN / 2 : WTN) * 2));
+    else
+        tile_epilogue<T, WTM, WTN, SWIGLU>(acc, Bias, Y, mt, N, ncols, n0, wm, wn, lane);
+}
+
+template <typename T, int BM, int BN, int WM, int WN>
 int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
-                 int64_t N, int epilogue, void *Y, hipStream_t s)
+                   int64_t N, int epilogue, void *Y, hipStream_t s)
 {
     constexpr int smem = 2 * (BM + BN) * ROWB;
     const bool sw = epilogue == OPMX_EPILOGUE_SWIGLU;
     const int64_t ncols = sw ? N / 2 : N;
     const int ntiles_n = static_cast<int>(ceil_div(ncols, sw ? BN / 2 : BN));
     const int ntiles_m = static_cast<int>(max_mtiles(R, E, BM));
-    // XCD-grouped order only when the n-tiles split evenly over the 8 XCDs (else some XCDs idle)
-    int gnx = ntiles_n % 16 == 0 ? 2 : (ntiles_n % 8 == 0 ? 1 : 0);
-    if (const char *v = std::getenv("OPMX_MOE_GEMM_GNX")) gnx = std::atoi(v);   // tuning knob (0: row-major)
-    if (gnx != 0 && gnx != 1 && gnx != 2 && gnx != 4 && gnx != 8 && gnx != 16 && gnx != 32) gnx = 0;
-    const int64_t nblocks = gnx > 0 ? ceil_div(ntiles_n, 8 * gnx) * ceil_div(ntiles_m, 32 / gnx) * 256
-                                    : static_cast<int64_t>(ntiles_n) * ntiles_m;
+    const int gnx = pick_gnx(ntiles_n);
+    const int64_t nblocks = linear_ids(gnx, ntiles_m, ntiles_n);
     dim3 grid(static_cast<unsigned>(nblocks));
     dim3 block(WM * WN * 64);
     static bool attr_done[2] = {false, false};
     if (sw) {
-        auto kern = gemm_tiled_kernel<T, BM, BN, WM, WN, true, ILV>;
+        auto kern = gemm_tiled_kernel<T, BM, BN, WM, WN, true>;
         if (!attr_done[1]) {
             if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                     smem) != hipSuccess)
@@ -278,9 +688,9 @@ int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B
             attr_done[1] = true;
         }
         kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
-                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_m, ntiles_n, gnx);
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_n, gnx);
     } else {
-        auto kern = gemm_tiled_kernel<T, BM, BN, WM, WN, false, ILV>;
+        auto kern = gemm_tiled_kernel<T, BM, BN, WM, WN, false>;
         if (!attr_done[0]) {
             if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                     smem) != hipSuccess)
@@ -288,7 +698,46 @@ int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B
             attr_done[0] = true;
         }
         kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
-                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_m, ntiles_n, gnx);
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_n, gnx);
+    }
+    OPMX_LAUNCH_CHECK();
+    return OPMX_OK;
+}
+
+template <typename T, int BM, int BN>
+int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
+                       int64_t K, int64_t N, int epilogue, void *Y, hipStream_t s)
+{
+    constexpr int smem = 2 * (BM + BN) * ROWB;
+    const bool sw = epilogue == OPMX_EPILOGUE_SWIGLU;
+    const int64_t ncols = sw ? N / 2 : N;
+    const int ntiles_n = static_cast<int>(ceil_div(ncols, sw ? BN / 2 : BN));
+    const int ntiles_m = static_cast<int>(max_mtiles(R, E, BM));
+    const int gnx = pick_gnx(ntiles_n);
+    const int64_t nblocks = linear_ids(gnx, ntiles_m, ntiles_n);
+    dim3 grid(static_cast<unsigned>(nblocks));
+    dim3 block(256);
+    static bool attr_done[2] = {false, false};
+    if (sw) {
+        auto kern = gemm_tiled_dlds_kernel<T, BM, BN, true>;
+        if (!attr_done[1]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    smem) != hipSuccess)
+                return OPMX_ERR_LAUNCH;
+            attr_done[1] = true;
+        }
+        kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_n, gnx);
+    } else {
+        auto kern = gemm_tiled_dlds_kernel<T, BM, BN, false>;
+        if (!attr_done[0]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    smem) != hipSuccess)
+                return OPMX_ERR_LAUNCH;
+            attr_done[0] = true;
+        }
+        kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_n, gnx);
     }
     OPMX_LAUNCH_CHECK();
     return OPMX_OK;
@@ -298,14 +747,10 @@ template <typename T>
 int tiled_impl(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
                int64_t N, int epilogue, int variant, void *Y, hipStream_t s)
 {
-    // The fixed MFMA / LDS / global-load interleave pays on the 256x256 tiles only.
     switch (variant) {
-        case 1: return tiled_launch<T, 256, 256, 2, 2, true>(X, off, W, B, E, R, K, N, epilogue, Y, s);
-        case 2: return tiled_launch<T, 256, 128, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
-        case 3: return tiled_launch<T, 256, 256, 2, 4, true>(X, off, W, B, E, R, K, N, epilogue, Y, s);
-        case 4: return tiled_launch<T, 256, 128, 4, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
-        case 5: return tiled_launch<T, 128, 256, 2, 4>(X, off, W, B, E, R, K, N, epilogue, Y, s);
-        default: return tiled_launch<T, 128, 128, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        case 1: return tiled_launch<T, 256, 256, 2, 4>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        case 2: return tiled_launch<T, 128, 128, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        default: return tiled_dlds_launch<T, 256, 256>(X, off, W, B, E, R, K, N, epilogue, Y, s);
     }
 }
 
@@ -313,7 +758,7 @@ int tiled_impl(const void *X, const int64_t *off, const void *W, const void *B, 
 
 // Requires: dtype f16/bf16, K % 64 == 0, 16-byte aligned X and W, N*K < 2^31.
 int launch_gemm_tiled(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
-                      int64_t K, int64_t N, int dtype, int epilogue, int variant, void *Y, hipStream_t s)
+                        int64_t K, int64_t N, int dtype, int epilogue, int variant, void *Y, hipStream_t s)
 {
     switch (dtype) {
         case OPMX_DTYPE_F16: return tiled_impl<f16>(X, off, W, B, E, R, K, N, epilogue, variant, Y, s);

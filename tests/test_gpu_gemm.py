@@ -83,7 +83,7 @@ def test_tiny_config_fp32_shapes():
     run_case("column", sizes, 1024, 5632, torch.float32, True, swiglu=True)
 
 
-@pytest.mark.parametrize("variant", ["0", "1", "2", "3", "4", "5", "6", "7", "8", "9", "10", "11", "12", "13", "14"])
+@pytest.mark.parametrize("variant", ["0", "1", "2"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_tiled_kernel_variants(variant, dtype):
     env = {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": variant}
@@ -95,7 +95,7 @@ def test_tiled_kernel_variants(variant, dtype):
     run_case("column", sizes, 64, 1000, dtype, False, env, swiglu=True)   # D=500: ragged epilogue tile
 
 
-@pytest.mark.parametrize("variant", ["7", "10", "11", "12", "13", "14"])
+@pytest.mark.parametrize("variant", ["0", "1", "2"])
 def test_tile_order_with_partial_last_round(variant):
     """16 column tiles and 24 row tiles: one full 16 x 16 round in the XCD-grouped order plus
     eight row tiles dealt out by the remainder rule; SwiGLU case: 16 column tiles of 128."""
