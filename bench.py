@@ -14,6 +14,9 @@ already resident in HBM.  Prints ONE JSON line:
   per_op_us            mean duration of each operator (separate untimed pass)
   device_ceilings      streaming-read GB/s and MFMA TFLOP/s (random fp16 operands) this
                        device sustains, from the probe ppl.pmx_amd/lib/opmx_device_ceilings
+  vendor_dense_gemm_same_flops_TFLOPs
+                       MFMA-bound workloads: the vendor library's dense GEMM with the flop
+                       count of the gate/up launch (no expert grouping), context only
   cpu_baseline         the CPU oracle (PyTorch CPU restatement of the reference
                        operator sequence) on the host cores, bounded sample
 
@@ -41,7 +44,7 @@ MFMA_PEAK_TFLOPS = 2500.0      # dense fp16/bf16 MFMA, vendor figure
 # profiles/gemm_tiled_prefill_T8192_mixtral8x7b.txt.  None where no counter run was made.
 MEASURED_TRAFFIC = {
     ("decode-T32", False): 1883442790 + 3759718,
-    ("prefill-T8192", False): 2 * 5360842 * 1024 + 927043 * 1024,
+    ("prefill-T8192", False): 2 * 3569692 * 1024 + 917504 * 1024,
 }
 
 SHAPES = {
@@ -71,6 +74,8 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg")
     ap.add_argument("--no-device-ceilings", action="store_true",
                     help="skip the probe of the HBM-read / MFMA rates this device sustains")
+    ap.add_argument("--no-vendor-gemm", action="store_true",
+                    help="MFMA-bound workloads: skip timing the vendor dense GEMM of the same flop count")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
                     help="also run N plain device-to-device copies of the gate/up weight tensor (known size): "
                          "the reference reading for FETCH_SIZE / WRITE_SIZE counter runs")
@@ -182,6 +187,24 @@ def main():
             for name, a, b in rec:
                 per_op[name] = per_op.get(name, 0.0) + a.elapsed_time(b) * 1e3 / reps
 
+    # Context for MFMA-bound workloads: the vendor library's dense GEMM (hipBLASLt behind
+    # torch.nn.functional.linear) on [R, H] x [2I, H]^T, the flop count of the gate/up launch
+    # without expert grouping or ragged tiles, same random operands, measured the same way.
+    vendor_tflops = None
+    if cfg["kind"] != "decode" and T >= 1024 and not args.no_vendor_gemm:
+        with torch.inference_mode():
+            xe_d = torch.randn(T * k, H, generator=g, device=dev).to(dtype)
+            for _ in range(3):
+                torch.nn.functional.linear(xe_d, wu[0])
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(10):
+                torch.nn.functional.linear(xe_d, wu[0])
+            b.record()
+            torch.cuda.synchronize()
+            vendor_tflops = round(2.0 * T * k * H * 2 * I / (a.elapsed_time(b) / 10 * 1e-3) / 1e12, 1)
+            del xe_d
+
     if args.copy_calibration > 0:
         dst = torch.empty_like(wu)
         for _ in range(args.copy_calibration):
@@ -222,7 +245,7 @@ def main():
         if hbm_bound:
             roof["measured_ceiling"] = ceilings["hbm_read_nontemporal_GBs"]
         else:
-            roof["measured_ceiling"] = ceilings["mfma_f16_lds_fed_TFLOPs"]
+            roof["measured_ceiling"] = ceilings.get("mfma_f16_16x16x32_lds_fed_TFLOPs", ceilings["mfma_f16_lds_fed_TFLOPs"])
         roof["frac_of_measured_ceiling"] = round(roof["achieved"] / roof["measured_ceiling"], 4)
 
     result = {
@@ -236,7 +259,7 @@ def main():
             "path": "drop-in operator sequence" + (" + fused SwiGLU epilogue" if args.fuse_swiglu else ""),
             "active_experts": active, "max_expert_share": round(float(counts.max()) / R, 3)},
         "roofline": roof, "layer": lay, "per_op_us": {n: round(v, 1) for n, v in per_op.items()},
-        "device_ceilings": ceilings, "device": torch.cuda.get_device_name(0), "cu_count": torch.cuda.get_device_properties(0).multi_processor_count,
+        "device_ceilings": ceilings, "vendor_dense_gemm_same_flops_TFLOPs": vendor_tflops, "device": torch.cuda.get_device_name(0), "cu_count": torch.cuda.get_device_properties(0).multi_processor_count,
     }
 
     # ---- CPU baseline: the oracle (PyTorch CPU restatement of the reference operator

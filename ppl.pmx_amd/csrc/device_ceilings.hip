@@ -1,6 +1,6 @@
 // Device-ceiling probe for MI355X: what this GPU sustains for (a) a pure streaming
-// read of a weight-sized buffer and (b) an MFMA loop on random fp16 operands,
-// register-fed and LDS-fed.  These are the practical ceilings the grouped-GEMM
+// read of a weight-sized buffer and (b, c) MFMA loops (32x32x16 and 16x16x32) on random fp16
+// operands, register-fed and LDS-fed.  These are the practical ceilings the grouped-GEMM
 // kernels are compared with in addition to the vendor peaks (8 TB/s, 2.5 PFLOP/s):
 // the engine clock drops under dense MFMA load with toggling operands, so the vendor
 // MFMA peak is not reachable by any kernel on real data.
@@ -79,6 +79,48 @@ __global__ __launch_bounds__(512) void mfma_kernel(const _Float16 *__restrict__ 
     out[blockIdx.x * blockDim.x + tid] = s;
 }
 
+// ---- (c) the same for MFMA 16x16x32 f16 (the grouped-GEMM kernels' instruction); LDS_FED:
+// 12 ds_read_b128 per 32 MFMAs, the same fragment bytes per flop as above
+typedef float float4v __attribute__((ext_vector_type(4)));
+template <bool LDS_FED>
+__global__ __launch_bounds__(512) void mfma16_kernel(const _Float16 *__restrict__ src, float *out, int iters)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int tid = threadIdx.x;
+    for (int i = tid; i < 65536 / 16; i += blockDim.x)
+        reinterpret_cast<u32x4 *>(smem)[i] = reinterpret_cast<const u32x4 *>(src)[i + (blockIdx.x & 7) * 4096];
+    __syncthreads();
+    float4v acc[32];
+    for (int j = 0; j < 32; ++j)
+        for (int v = 0; v < 4; ++v) acc[j][v] = 0.f;
+    const int base = (tid >> 6) * 4096 + (tid & 63) * 16;
+    half8 fa[2][8], fb[2][4];
+    auto rd = [&](int set, int it) {
+        const int o = (base + (it & 15) * 3072) & 65520;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) fa[set][i] = *reinterpret_cast<const half8 *>(smem + ((o + i * 1024) & 65535));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) fb[set][i] = *reinterpret_cast<const half8 *>(smem + ((o + 32768 + i * 1024) & 65535));
+    };
+    rd(0, 0);
+    rd(1, 1);
+    for (int it = 0; it < iters; it += 2) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            if (LDS_FED) rd((h + 1) & 1, it + h + 1);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[i * 4 + j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa[h][i], fb[h][j], acc[i * 4 + j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    float s = 0;
+    for (int j = 0; j < 32; ++j) s += acc[j][0] + acc[j][3];
+    out[blockIdx.x * blockDim.x + tid] = s;
+}
+
 static float best_ms(hipEvent_t e0, hipEvent_t e1, int reps, void (*launch)(void *), void *ctx)
 {
     float best = 1e30f;
@@ -95,7 +137,7 @@ static float best_ms(hipEvent_t e0, hipEvent_t e1, int reps, void (*launch)(void
 }
 
 struct ReadCtx { const u32x4 *src; size_t n16; unsigned *out; int blocks; bool nt; };
-struct MfmaCtx { const _Float16 *src; float *out; int iters; bool lds; };
+struct MfmaCtx { const _Float16 *src; float *out; int iters; bool lds; bool m16; };
 
 int main()
 {
@@ -133,19 +175,37 @@ int main()
                               hipFuncAttributeMaxDynamicSharedMemorySize, 65536));
     CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(mfma_kernel<false>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, 65536));
-    MfmaCtx mc{src, out, 8000, false};
+    CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(mfma16_kernel<true>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 65536));
+    CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(mfma16_kernel<false>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 65536));
+    MfmaCtx mc{src, out, 8000, false, false};
     auto mfma_launch = [](void *c) {
         MfmaCtx *m = static_cast<MfmaCtx *>(c);
-        if (m->lds) mfma_kernel<true><<<256, 512, 65536>>>(m->src, m->out, m->iters);
-        else mfma_kernel<false><<<256, 512, 65536>>>(m->src, m->out, m->iters);
+        if (m->m16) {
+            if (m->lds) mfma16_kernel<true><<<256, 512, 65536>>>(m->src, m->out, m->iters);
+            else mfma16_kernel<false><<<256, 512, 65536>>>(m->src, m->out, m->iters);
+        } else {
+            if (m->lds) mfma_kernel<true><<<256, 512, 65536>>>(m->src, m->out, m->iters);
+            else mfma_kernel<false><<<256, 512, 65536>>>(m->src, m->out, m->iters);
+        }
     };
     const double flops = 256.0 * 8 * mc.iters * 8 * 32768.0;
     const double mfma_reg = flops / best_ms(e0, e1, 5, mfma_launch, &mc) / 1e9;
     mc.lds = true;
     const double mfma_lds = flops / best_ms(e0, e1, 5, mfma_launch, &mc) / 1e9;
+    // 16x16x32: 32 MFMAs of 16384 flops per iteration, same flops per iteration count as above
+    mc.m16 = true;
+    mc.lds = false;
+    mc.iters = 4000;
+    const double flops16 = 256.0 * 8 * mc.iters * 32 * 16384.0;
+    const double mfma16_reg = flops16 / best_ms(e0, e1, 5, mfma_launch, &mc) / 1e9;
+    mc.lds = true;
+    const double mfma16_lds = flops16 / best_ms(e0, e1, 5, mfma_launch, &mc) / 1e9;
     CHECK(hipGetLastError());
     printf("{\"hbm_read_GBs\": %.0f, \"hbm_read_nontemporal_GBs\": %.0f, "
-           "\"mfma_f16_register_fed_TFLOPs\": %.0f, \"mfma_f16_lds_fed_TFLOPs\": %.0f}\n",
-           read_plain, read_nt, mfma_reg, mfma_lds);
+           "\"mfma_f16_register_fed_TFLOPs\": %.0f, \"mfma_f16_lds_fed_TFLOPs\": %.0f, "
+           "\"mfma_f16_16x16x32_register_fed_TFLOPs\": %.0f, \"mfma_f16_16x16x32_lds_fed_TFLOPs\": %.0f}\n",
+           read_plain, read_nt, mfma_reg, mfma_lds, mfma16_reg, mfma16_lds);
     return 0;
 }
