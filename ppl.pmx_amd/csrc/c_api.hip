@@ -39,14 +39,17 @@ int forced_kernel()
 
 namespace opmx {
 
+// Scratch memory that lets the 256x256 tile kernel balance its last rounds of tiles over all
+// CUs (stream-K); every kernel also runs without it.  256 bytes when the call would not use it.
 size_t grouped_gemm_workspace_bytes(int E, int64_t R, int64_t K, int64_t N, int dtype)
 {
-    (void)E;
-    (void)R;
-    (void)K;
     (void)N;
-    (void)dtype;
-    return 256;   // every epilogue is applied in registers; the argument is kept for ABI stability
+    const bool lowp = dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16;
+    if (lowp && E > 0 && K > 0 && K % 64 == 0 && R / E >= 128) {
+        const size_t b = gemm_tiled_workspace_bytes();
+        if (b > 0) return (b + 255) / 256 * 256;
+    }
+    return 256;
 }
 
 int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
@@ -64,9 +67,7 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
     int64_t hint = rows_hint > 0 && rows_hint < R ? rows_hint : R;
     const int64_t twice_mean = 2 * ceil_div(R, E);
     if (twice_mean < hint) hint = twice_mean;
-    (void)ws;
-    (void)ws_bytes;
-    const bool stream_ws = true;   // no kernel needs scratch memory today
+    const bool stream_ws = true;   // the stream kernel needs no scratch memory
     const int force = forced_kernel();
 
     int choice;   // 1 generic, 2 tiled, 3 stream
@@ -84,7 +85,7 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
         // 256x256 direct-to-LDS tiles from 128 mean rows per expert on, else 128x128 (measured).
         const int dflt = R / E >= 128 ? 0 : 2;
         return launch_gemm_tiled(X, off, W, B, E, R, K, N, dtype, epilogue,
-                                 env_int("OPMX_MOE_GEMM_TILED_VARIANT", dflt), Y, s);
+                                 env_int("OPMX_MOE_GEMM_TILED_VARIANT", dflt), Y, ws, ws_bytes, s);
     }
     return launch_gemm_generic(X, off, W, B, E, R, K, N, dtype, epilogue, Y, s);
 }

@@ -128,8 +128,12 @@ int launch_gemm_generic(const void *X, const int64_t *off, const void *W, const 
                         int64_t K, int64_t N, int dtype, int epilogue, void *Y, hipStream_t s);
 // variant: 0 = 256x256 direct-to-LDS kernel, 1 = 256x256 register-staged (8 waves),
 // 2 = 128x128 register-staged (4 waves).  off == nullptr: dense GEMM (one expert owns [0, R)).
+// ws / ws_bytes: optional scratch memory of gemm_tiled_workspace_bytes() bytes (variant 0 then
+// balances the last rounds of tiles over all CUs); nullptr / 0 is always accepted.
 int launch_gemm_tiled(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
-                      int64_t K, int64_t N, int dtype, int epilogue, int variant, void *Y, hipStream_t s);
+                      int64_t K, int64_t N, int dtype, int epilogue, int variant, void *Y, void *ws,
+                      size_t ws_bytes, hipStream_t s);
+size_t gemm_tiled_workspace_bytes();
 int launch_gemm_stream(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
                        int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint, int variant, void *Y,
                        hipStream_t s);

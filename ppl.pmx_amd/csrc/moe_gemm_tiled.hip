@@ -103,17 +103,16 @@ __device__ __forceinline__ void map_tile(int lin, int gnx, int mtiles, int ntile
     }
 }
 
-// Linear tile id -> (row tile of one expert, column tile).  mt.rows == 0 when the id names no
-// work.  s_off: see stage_offsets (unused when `grouped` is false: one expert owns [0, R)).
-__device__ __forceinline__ void locate_tile(int lin, int gnx, int mtiles, int ntiles_n, bool grouped,
-                                            const int64_t *s_off, int E, int64_t R, int BM, MTile &mt, int &tile_n)
+// Row tile tile_m (counted over all experts in expert order) -> expert and row range.
+// mt.rows == 0 when there is no such tile.  s_off: see stage_offsets (unused when `grouped` is
+// false: one expert owns [0, R)).
+__device__ __forceinline__ void row_tile(int tile_m, bool grouped, const int64_t *s_off, int E, int64_t R, int BM,
+                                         MTile &mt)
 {
-    int tile_m;
-    map_tile(lin, gnx, mtiles, ntiles_n, tile_m, tile_n);
     mt.e = 0;
     mt.rows = 0;
     mt.row0 = 0;
-    if (tile_m >= mtiles || tile_n >= ntiles_n) return;
+    if (tile_m < 0) return;
     if (!grouped) {
         mt.row0 = static_cast<int64_t>(tile_m) * BM;
         const int64_t left = R - mt.row0;
@@ -137,6 +136,16 @@ __device__ __forceinline__ void locate_tile(int lin, int gnx, int mtiles, int nt
         tile -= nt;
         prev = hi;
     }
+}
+
+// Linear tile id -> (row tile of one expert, column tile).  mt.rows == 0 when the id names no work.
+__device__ __forceinline__ void locate_tile(int lin, int gnx, int mtiles, int ntiles_n, bool grouped,
+                                            const int64_t *s_off, int E, int64_t R, int BM, MTile &mt, int &tile_n)
+{
+    int tile_m;
+    map_tile(lin, gnx, mtiles, ntiles_n, tile_m, tile_n);
+    if (tile_m >= mtiles || tile_n >= ntiles_n) tile_m = -1;
+    row_tile(tile_m, grouped, s_off, E, R, BM, mt);
 }
 
 // Host side of map_tile: the order to use and the number of linear ids it spans.
@@ -486,6 +495,30 @@ __device__ __forceinline__ void load_to_lds_16(__amdgpu_buffer_rsrc_t r, char *l
     __builtin_amdgcn_raw_ptr_buffer_load_lds(r, OPMX_LPTR(lds), 16, voff, soff, 0, 0);
 }
 
+// Tail balancing ("split-K of the last round").  With G workgroup slots (one per CU) the last
+// ttot % G tiles of the row-major tile order would run alone on a mostly idle chip.  When the
+// caller lends scratch memory they are left to a second launch in which each of them is cut
+// into `g` equal k-ranges, one workgroup each; the partial sums meet in the scratch memory.
+// In the 2-D tile order (gnx = 4; the split is used with no other) the tile ids are exactly
+// [0, ttot) and the tail ids are spread evenly over the XCDs; XCD j keeps the tail tiles it would
+// have had (ids = j mod 8: a compact block of the tile grid) with all their k-ranges, so its
+// workgroups walk the same k positions at the same time and keep sharing X- and W-tiles in L2.  g = 1: no split, the one-tile-per-workgroup launch does
+// everything.  Must give the same answer on the host and on the device.
+__host__ __device__ inline int sk_split(int64_t ttot, int sk_wgs, int nk, int gnx, int cost)
+{
+    if (sk_wgs < 8 || gnx != 4) return 1;
+    const int64_t tail = ttot % sk_wgs;
+    if (tail == 0) return 1;
+    const int per_xcd = static_cast<int>((tail + 7) / 8);
+    int g = (sk_wgs / 8) / per_xcd;
+    if (g > nk / 8) g = nk / 8;          // at least 8 k-tiles per range
+    if (g > 8) g = 8;
+    if (g < 2) return 1;
+    // the exchange of partial sums costs about as much as `cost` k-tiles of work; split only when
+    // the time saved, (1 - 1/g) of a tile, is more
+    return (g - 1) * nk > cost * g ? g : 1;
+}
+
 // ---------------------------------------------------------------------------------------
 // Direct-to-LDS, 4 waves, fragments of a whole k-tile held in registers.  Each wave reads all
 // 32 fragments of k-tile kt (128 VGPRs) by the first third of the k-tile, so the LDS buffer is
@@ -498,13 +531,37 @@ __device__ __forceinline__ void load_to_lds_16(__amdgpu_buffer_rsrc_t r, char *l
 //     group 3 reads the first fragments of k-tile kt+1.
 // MFMAs are volatile asm (accumulators pinned to the 256 accumulation registers), so the
 // source order below is the issue order.
-template <typename T, int BM, int BN, bool SWIGLU>
+// Partial sums cross XCDs (each has its own L2).  16-byte buffer accesses with the device-scope
+// cache policy (sc0 sc1) write through to / read from the coherent level, which avoids the
+// whole-L2 write-back and invalidate that a device-scope fence costs on this part; ordering
+// against the arrival counter is by waiting for the stores (s_waitcnt vmcnt(0)) before the
+// block barrier that precedes the counter update.  `slot` describes one fp32 tile-sized slot,
+// `idx` counts 16-byte elements in it.
+constexpr int kDeviceScope = 17;   // sc0 | sc1
+__device__ __forceinline__ void coherent_store(__amdgpu_buffer_rsrc_t slot, int idx, float4_t v)
+{
+    u32x4 bits;
+    __builtin_memcpy(&bits, &v, 16);
+    __builtin_amdgcn_raw_buffer_store_b128(bits, slot, idx * 16, 0, kDeviceScope);
+}
+__device__ __forceinline__ float4_t coherent_load(__amdgpu_buffer_rsrc_t slot, int idx)
+{
+    const u32x4 bits = __builtin_amdgcn_raw_buffer_load_b128(slot, idx * 16, 0, kDeviceScope);
+    float4_t v;
+    __builtin_memcpy(&v, &bits, 16);
+    return v;
+}
+
+// SK = false: one tile per workgroup (all tiles, or all but the tail when sk_wgs > 0 and the
+// tail is split).  SK = true: the tail launch, one k-range of one tail tile per workgroup.
+template <typename T, int BM, int BN, bool SWIGLU, bool SK>
 __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restrict__ X,
                                                                const int64_t *__restrict__ off,
                                                                const T *__restrict__ W,
                                                                const T *__restrict__ Bias, int E, int64_t R,
                                                                int64_t K, int64_t N, T *__restrict__ Y,
-                                                               int ntiles_n, int gnx)
+                                                               int ntiles_n, int gnx, int sk_wgs, int sk_cost,
+                                                               float *__restrict__ sk_part, int *__restrict__ sk_count)
 {
     constexpr int WM = 2, WN = 2, NW = 4;
     constexpr int WTM = BM / WM, WTN = BN / WN, TMS = WTM / 16, TNS = WTN / 16, HM = TMS / 2;
@@ -518,13 +575,43 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
     extern __shared__ __attribute__((aligned(16))) char smem[];
     __shared__ int64_t s_off[OPMX_MOE_MAX_EXPERTS + 1];
 
+    __shared__ int s_arrivals;
     const int64_t ncols = SWIGLU ? N / 2 : N;
-    zero_unowned_rows(Y, R, ncols, off, E);
+    if (!SK) zero_unowned_rows(Y, R, ncols, off, E);
     stage_offsets(off, E, R, s_off);
+    const int mtiles = count_mtiles(off != nullptr, s_off, E, R, BM);
+    const int nk = static_cast<int>(K / BK);
+    const int64_t ttot = static_cast<int64_t>(mtiles) * ntiles_n;
+    const int g = sk_split(ttot, sk_wgs, nk, gnx, sk_cost);
+    const int64_t tail = g > 1 ? ttot % sk_wgs : 0;      // tiles left to the tail launch
     MTile mt;
-    int tile_n;
-    locate_tile(blockIdx.x, gnx, count_mtiles(off != nullptr, s_off, E, R, BM), ntiles_n, off != nullptr, s_off, E, R,
-                BM, mt, tile_n);
+    int tile_m, tile_n;
+    int kt0 = 0, kt1 = nk;          // k-tiles of this workgroup
+    int tail_tile = 0, chunk = 0;   // SK: which tail tile, which of its g k-ranges
+    int xcd_first = 0, xcd_tiles = 0;
+    if (!SK) {
+        // with the 2-D order (the only one the tail split is used with) the ids [0, ttot) are
+        // exactly the tiles, and the last `tail` of them are spread evenly over the XCDs
+        if (static_cast<int64_t>(blockIdx.x) >= ttot - tail && tail > 0) return;
+        map_tile(blockIdx.x, gnx, mtiles, ntiles_n, tile_m, tile_n);
+        if (tile_m >= mtiles || tile_n >= ntiles_n) return;
+    } else {
+        if (tail == 0) return;
+        // XCD j (workgroups j, j+8, ...) takes the tail ids congruent to j mod 8 -- the tiles it
+        // would have had in the other launch, a compact block of the tile grid -- with all their
+        // k-ranges: position p = range * tiles + tile
+        const int xcd = blockIdx.x & 7, p = blockIdx.x >> 3;
+        const int64_t base = ttot - tail;
+        xcd_first = static_cast<int>((xcd - base) & 7);                    // first tail tile of this XCD
+        xcd_tiles = xcd_first < tail ? static_cast<int>((tail - xcd_first + 7) / 8) : 0;
+        if (p >= xcd_tiles * g) return;
+        chunk = p / xcd_tiles;
+        tail_tile = xcd_first + 8 * (p % xcd_tiles);
+        kt0 = chunk * nk / g;
+        kt1 = (chunk + 1) * nk / g;
+        map_tile(static_cast<int>(base + tail_tile), gnx, mtiles, ntiles_n, tile_m, tile_n);
+    }
+    row_tile(tile_m, off != nullptr, s_off, E, R, BM, mt);
     if (mt.rows == 0) return;
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -569,7 +656,6 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
 #pragma unroll
             for (int v = 0; v < 4; ++v) acc[j][i][v] = 0.0f;
 
-    const int nk = static_cast<int>(K / BK);
     const int lrow = lane & 15, lk = lane >> 4;
     const int swz = (lrow >> 1) & 7;
     const int x_off = (wm * WTM + lrow) * ROWB;
@@ -623,12 +709,12 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
         }                                                                                          \
     } while (0)
 
-    // prologue: k-tile 0 -> buffer 0, k-tile 1 -> buffer 1, wait for k-tile 0
+    // prologue: first k-tile -> buffer 0, second -> buffer 1, wait for the first
 #pragma unroll
-    for (int q = 0; q < NL; ++q) OPMX_ISSUE1(0, 0, q);
-    if (nk > 1) {
+    for (int q = 0; q < NL; ++q) OPMX_ISSUE1(kt0, 0, q);
+    if (kt1 - kt0 > 1) {
 #pragma unroll
-        for (int q = 0; q < NL; ++q) OPMX_ISSUE1(1, 1, q);
+        for (int q = 0; q < NL; ++q) OPMX_ISSUE1(kt0 + 1, 1, q);
         asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
     } else {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -640,9 +726,9 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
 #pragma unroll
     for (int j = 0; j < TNS; ++j) OPMX_WFRAG(0, 0, j);
     {
-        int kt = 0, b = 0;
-        for (; kt + 2 < nk; ++kt, b ^= 1) OPMX_ITER(kt, b, true, true);
-        if (kt + 1 < nk) {
+        int kt = kt0, b = 0;
+        for (; kt + 2 < kt1; ++kt, b ^= 1) OPMX_ITER(kt, b, true, true);
+        if (kt + 1 < kt1) {
             OPMX_ITER(kt, b, false, true);
             ++kt;
             b ^= 1;
@@ -657,12 +743,57 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
 
     // asm MFMAs are opaque to the compiler's hazard padding: let the last ones retire
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+
+    if (SK) {
+        // A k-range of a tail tile.  Every workgroup parks its fp32 partial sums in its own slot
+        // and adds its number of k-tiles to the tile's counter; the one that completes the count
+        // adds all g partial sums up in k order (so the result does not depend on who was last)
+        // and writes the tile.
+        const __amdgpu_buffer_rsrc_t mine = raw_descriptor(sk_part + static_cast<int64_t>(blockIdx.x) * (BM * BN));
+#pragma unroll
+        for (int j = 0; j < TNS; ++j)
+#pragma unroll
+            for (int i = 0; i < TMS; ++i) coherent_store(mine, (j * TMS + i) * 256 + tid, acc[j][i]);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0)
+            s_arrivals = __hip_atomic_fetch_add(sk_count + tail_tile, kt1 - kt0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (s_arrivals + (kt1 - kt0) != nk) return;          // not the last one (uniform)
+#pragma unroll
+        for (int j = 0; j < TNS; ++j)
+#pragma unroll
+            for (int i = 0; i < TMS; ++i)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc[j][i][v] = 0.0f;
+        // the slot of k-range c of this tile: workgroup (this XCD, position c*tiles + tile)
+        for (int c = 0; c < g; ++c) {
+            const int wg = ((c * xcd_tiles + ((tail_tile - xcd_first) >> 3)) << 3) + (blockIdx.x & 7);
+            const __amdgpu_buffer_rsrc_t theirs = raw_descriptor(sk_part + static_cast<int64_t>(wg) * (BM * BN));
+            // sixteen loads in flight at a time: one at a time would be 64 serial round trips
+#pragma unroll
+            for (int blk = 0; blk < TNS * TMS / 16; ++blk) {
+                float4_t part[16];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) part[u] = coherent_load(theirs, (blk * 16 + u) * 256 + tid);
+#pragma unroll
+                for (int u = 0; u < 16; ++u) acc[(blk * 16 + u) / TMS][(blk * 16 + u) % TMS] += part[u];
+            }
+        }
+    }
     // after the last barrier no wave reads operand tiles any more: LDS is free for the epilogue
     if (ncols % 8 == 0 && reinterpret_cast<uintptr_t>(Y) % 16 == 0)
         tile_epilogue_lds<T, WTM, WTN, SWIGLU>(acc, Bias, Y, mt, N, ncols, n0, wm, wn, lane,
                                                smem + wave * (WTM * (SWIGLU ? WTN / 2 : WTN) * 2));
     else
         tile_epilogue<T, WTM, WTN, SWIGLU>(acc, Bias, Y, mt, N, ncols, n0, wm, wn, lane);
+}
+
+// Clears the arrival counters of the tail tiles (a kernel, not a memset: callers may capture
+// the launch sequence in a graph).
+__global__ void sk_clear_kernel(int *__restrict__ count, int n)
+{
+    for (int i = threadIdx.x; i < n; i += blockDim.x) count[i] = 0;
 }
 
 template <typename T, int BM, int BN, int WM, int WN>
@@ -704,40 +835,87 @@ int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B
     return OPMX_OK;
 }
 
+// Scratch memory of the tail launch of the direct-to-LDS kernel.
+constexpr int kSkCounters = 256;                  // tail tiles are fewer than the CUs
+constexpr int kSkTile = 256 * 256;                // elements of an output tile
+
+int cu_count()
+{
+    static int num_cu = 0;
+    if (num_cu == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            return 0;
+        num_cu = n;
+    }
+    return num_cu;
+}
+
+// arrival counters, then one fp32 tile-sized slot per workgroup of the tail launch
+size_t sk_workspace_bytes(int cus)
+{
+    return static_cast<size_t>(kSkCounters) * sizeof(int) + static_cast<size_t>(cus) * kSkTile * sizeof(float);
+}
+
 template <typename T, int BM, int BN>
 int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
-                       int64_t K, int64_t N, int epilogue, void *Y, hipStream_t s)
+                      int64_t K, int64_t N, int epilogue, void *Y, void *ws, size_t ws_bytes, hipStream_t s)
 {
+    static_assert(BM * BN == kSkTile, "tail slot size");
     constexpr int smem = 2 * (BM + BN) * ROWB;
     const bool sw = epilogue == OPMX_EPILOGUE_SWIGLU;
     const int64_t ncols = sw ? N / 2 : N;
     const int ntiles_n = static_cast<int>(ceil_div(ncols, sw ? BN / 2 : BN));
     const int ntiles_m = static_cast<int>(max_mtiles(R, E, BM));
     const int gnx = pick_gnx(ntiles_n);
-    const int64_t nblocks = linear_ids(gnx, ntiles_m, ntiles_n);
-    dim3 grid(static_cast<unsigned>(nblocks));
+    const int64_t dp_ids = linear_ids(gnx, ntiles_m, ntiles_n);
+    if (dp_ids >= (int64_t{1} << 31)) return OPMX_ERR_UNSUPPORTED;
+    // split-K of the tail tiles when the caller lends the scratch memory for it.  The tile count
+    // is only known on the device, so the tail launch is always made; it exits at once when
+    // there is no tail or no split.
+    const int cus = cu_count();
+    int sk_wgs = 0;
+    if (ws != nullptr && cus >= 8 && cus % 8 == 0 && cus <= kSkCounters && ws_bytes >= sk_workspace_bytes(cus) &&
+        reinterpret_cast<uintptr_t>(ws) % 16 == 0 && gnx == 4)
+        sk_wgs = cus;
+    // Measured: the exchange costs ~100 us against 1.43 us per k-tile.
+    int sk_cost = 70;
+    if (const char *v = std::getenv("OPMX_MOE_GEMM_STREAMK")) {   // tuning knob: 0 = off, 2 = split whenever possible
+        if (std::atoi(v) == 0) sk_wgs = 0;
+        if (std::atoi(v) == 2) sk_cost = 0;
+    }
+    if (7 * (K / BK) <= 8 * sk_cost) sk_wgs = 0;     // sk_split() cannot split a K this short (g <= 8)
+    int *sk_count = static_cast<int *>(ws);
+    float *sk_part = reinterpret_cast<float *>(static_cast<char *>(ws) + kSkCounters * sizeof(int));
+    dim3 grid(static_cast<unsigned>(dp_ids));
     dim3 block(256);
     static bool attr_done[2] = {false, false};
+    if (!attr_done[sw ? 1 : 0]) {
+        const void *k1 = sw ? reinterpret_cast<const void *>(gemm_tiled_dlds_kernel<T, BM, BN, true, false>)
+                            : reinterpret_cast<const void *>(gemm_tiled_dlds_kernel<T, BM, BN, false, false>);
+        const void *k2 = sw ? reinterpret_cast<const void *>(gemm_tiled_dlds_kernel<T, BM, BN, true, true>)
+                            : reinterpret_cast<const void *>(gemm_tiled_dlds_kernel<T, BM, BN, false, true>);
+        if (hipFuncSetAttribute(k1, hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess ||
+            hipFuncSetAttribute(k2, hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess)
+            return OPMX_ERR_LAUNCH;
+        attr_done[sw ? 1 : 0] = true;
+    }
+    const T *Xp = static_cast<const T *>(X), *Wp = static_cast<const T *>(W), *Bp = static_cast<const T *>(B);
+    T *Yp = static_cast<T *>(Y);
+    if (sk_wgs > 0) sk_clear_kernel<<<1, 256, 0, s>>>(sk_count, kSkCounters);
     if (sw) {
-        auto kern = gemm_tiled_dlds_kernel<T, BM, BN, true>;
-        if (!attr_done[1]) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    smem) != hipSuccess)
-                return OPMX_ERR_LAUNCH;
-            attr_done[1] = true;
-        }
-        kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
-                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_n, gnx);
+        gemm_tiled_dlds_kernel<T, BM, BN, true, false><<<grid, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
+                                                                                 gnx, sk_wgs, sk_cost, sk_part, sk_count);
+        if (sk_wgs > 0)
+            gemm_tiled_dlds_kernel<T, BM, BN, true, true><<<sk_wgs, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
+                                                                                      gnx, sk_wgs, sk_cost, sk_part, sk_count);
     } else {
-        auto kern = gemm_tiled_dlds_kernel<T, BM, BN, false>;
-        if (!attr_done[0]) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    smem) != hipSuccess)
-                return OPMX_ERR_LAUNCH;
-            attr_done[0] = true;
-        }
-        kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
-                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_n, gnx);
+        gemm_tiled_dlds_kernel<T, BM, BN, false, false><<<grid, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
+                                                                                  gnx, sk_wgs, sk_cost, sk_part, sk_count);
+        if (sk_wgs > 0)
+            gemm_tiled_dlds_kernel<T, BM, BN, false, true><<<sk_wgs, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
+                                                                                       gnx, sk_wgs, sk_cost, sk_part, sk_count);
     }
     OPMX_LAUNCH_CHECK();
     return OPMX_OK;
@@ -745,26 +923,35 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
 
 template <typename T>
 int tiled_impl(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
-               int64_t N, int epilogue, int variant, void *Y, hipStream_t s)
+               int64_t N, int epilogue, int variant, void *Y, void *ws, size_t ws_bytes, hipStream_t s)
 {
     switch (variant) {
         case 1: return tiled_launch<T, 256, 256, 2, 4>(X, off, W, B, E, R, K, N, epilogue, Y, s);
         case 2: return tiled_launch<T, 128, 128, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
-        default: return tiled_dlds_launch<T, 256, 256>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        default: return tiled_dlds_launch<T, 256, 256>(X, off, W, B, E, R, K, N, epilogue, Y, ws, ws_bytes, s);
     }
 }
 
 }  // namespace
 
 // Requires: dtype f16/bf16, K % 64 == 0, 16-byte aligned X and W, N*K < 2^31.
+// ws / ws_bytes: optional scratch memory (gemm_tiled_workspace_bytes()); with it the default
+// variant balances the last rounds of tiles over all CUs.
 int launch_gemm_tiled(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
-                        int64_t K, int64_t N, int dtype, int epilogue, int variant, void *Y, hipStream_t s)
+                      int64_t K, int64_t N, int dtype, int epilogue, int variant, void *Y, void *ws,
+                      size_t ws_bytes, hipStream_t s)
 {
     switch (dtype) {
-        case OPMX_DTYPE_F16: return tiled_impl<f16>(X, off, W, B, E, R, K, N, epilogue, variant, Y, s);
-        case OPMX_DTYPE_BF16: return tiled_impl<bf16>(X, off, W, B, E, R, K, N, epilogue, variant, Y, s);
+        case OPMX_DTYPE_F16: return tiled_impl<f16>(X, off, W, B, E, R, K, N, epilogue, variant, Y, ws, ws_bytes, s);
+        case OPMX_DTYPE_BF16: return tiled_impl<bf16>(X, off, W, B, E, R, K, N, epilogue, variant, Y, ws, ws_bytes, s);
     }
     return OPMX_ERR_UNSUPPORTED;
+}
+
+size_t gemm_tiled_workspace_bytes()
+{
+    const int cus = cu_count();
+    return cus > 0 ? sk_workspace_bytes(cus) : 0;
 }
 
 }  // namespace opmx

@@ -36,11 +36,14 @@ def grouped_linear(op, X, expert_offset, W, B, num_experts, epilogue=_lib.EPILOG
     hint = R // X.shape[-2] if X.dim() >= 3 and X.shape[-2] > 0 else 0
     Y = torch.empty(R, n_out, dtype=W.dtype, device=dev)
     L = _lib.lib()
+    # optional scratch memory: with it the large-tile kernel balances its last rounds of tiles
+    # over all CUs; small calls report a token size and run without
     ws = None
-    ws_bytes = 0
-    if epilogue != _lib.EPILOGUE_NONE:
-        ws = _lib.workspace(L.opmx_moe_grouped_gemm_workspace_bytes(E, R, K, N, dt), dev)
-        ws_bytes = ws.numel()
+    ws_bytes = L.opmx_moe_grouped_gemm_workspace_bytes(E, R, K, N, dt)
+    if ws_bytes > 256:
+        ws = _lib.workspace(ws_bytes, dev)
+    else:
+        ws_bytes = 0
     if op == "column":
         rc = L.opmx_moe_column_parallel_linear(_lib.ptr(Xf), _lib.ptr(off), _lib.ptr(Wc), _lib.ptr(Bc), E, R, K, N,
                                                dt, epilogue, hint, _lib.ptr(Y), _lib.ptr(ws), ws_bytes,

@@ -106,6 +106,26 @@ def test_tile_order_with_partial_last_round(variant):
     run_case("row", [4096], 192, 4096, torch.float16, False, env)          # exactly one full round
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_tail_tiles_split_over_k(dtype):
+    """Few tiles (4 row tiles x 16 column tiles, 2-D tile order) and a long K: the tail launch of
+    the 256x256 kernel cuts every tile into k-ranges whose fp32 partial sums meet in the workspace
+    (K=2048: 4 ranges, K=1024: 2)."""
+    env = {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": "0", "OPMX_MOE_GEMM_STREAMK": "2"}   # 2: always split
+    sizes = [300, 77, 129]
+    a = run_case("row", sizes, 2048, 4096, dtype, True, env)
+    run_case("column", sizes, 1024, 4096, dtype, False, env, swiglu=True)     # 16 column tiles of 128
+    run_case("column", [700, 300, 1], 1024, 4096, dtype, False, env)          # 6 x 16 tiles
+    # same result bit for bit on a second call (summation order is fixed); close to the unsplit one
+    b = run_case("row", sizes, 2048, 4096, dtype, True, env)
+    assert torch.equal(a, b)
+    c = run_case("row", sizes, 2048, 4096, dtype, True, dict(env, OPMX_MOE_GEMM_STREAMK="0"))
+    assert (a.float() - c.float()).abs().max() <= 2e-2 * max(1.0, float(c.float().abs().max()))
+    # a K long enough for the default policy to split (144 k-tiles, 8 ranges)
+    if dtype == torch.float16:
+        run_case("row", [200, 60], 9216, 4096, dtype, False, {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": "0"})
+
+
 @pytest.mark.parametrize("variant", ["0", "1", "2", "3", "4", "5"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_stream_kernel_variants(variant, dtype):
