@@ -123,6 +123,15 @@ int opmx_swiglu(const void *X, int64_t R, int64_t D, float beta, int dtype, void
  *   Y[i] = gate[i] * X[i] * sigmoid(X[i])  (gate may be NULL);  n elements. */
 int opmx_silu(const void *X, const void *gate, int64_t n, int dtype, void *Y, void *stream);
 
+/* RMSNorm / SkipRMSNorm over the last dimension: the operator in front of the MoE layer
+ * (ffn_norm, model_zoo/mixtral/modeling/dynamic_batching/Model.py:261).  Replaces
+ * RMSNorm.forward and SkipRMSNorm.forward, torch_function/RMSNorm.py:16-24 and :44-56:
+ *   s = X + SkipIn (rounded to dtype; s = X when SkipIn is NULL)
+ *   Y = round(round(s * rsqrt(mean(s^2) + eps)) * weight),  SkipOut = s
+ * X, SkipIn, Y, SkipOut [T,H]; weight [H]; SkipOut may be NULL (plain RMSNorm). */
+int opmx_rms_norm(const void *X, const void *weight, const void *SkipIn, int64_t T, int64_t H, float eps,
+                  int dtype, void *Y, void *SkipOut, void *stream);
+
 /* MoeReduce.  Replaces MoeReduce.forward, torch_function/MoeReduce.py:16-26:
  *   out[t, :] = sum_{s<k} expert_weights[t,s] * Y[invert_permutation[t*k+s], :]
  * summed in slot order in fp32, rounded once.  Y [T*k,N], out [T,N].

@@ -14,6 +14,7 @@ Reference files restated (paths relative to the OpenPPL/ppl.pmx checkout):
 * ``torch_function/SiLU.py:18-21``                   -> :func:`silu`
 * ``torch_function/MoeRowParallelLinear.py:44-60``   -> :func:`moe_row_parallel_linear`
 * ``torch_function/MoeReduce.py:23-25``              -> :func:`moe_reduce`
+* ``torch_function/RMSNorm.py:16-24,44-56``          -> :func:`rms_norm`, :func:`skip_rms_norm`
 * ``model_zoo/mixtral/modeling/dynamic_batching/Model.py:187-214`` -> :func:`moe_layer`
 
 Third-party arithmetic: the reference delegates every number to PyTorch
@@ -204,6 +205,23 @@ def silu(X: torch.Tensor, gate: Optional[torch.Tensor] = None, acc=torch.float32
 # --------------------------------------------------------------------------
 # a6  MoeReduce                                          MoeReduce.py:23-25
 # --------------------------------------------------------------------------
+
+def skip_rms_norm(X, weight, SkipIn=None, eps=1e-5):
+    """SkipRMSNorm over the last axis with the reference's roundings
+    (torch_function/RMSNorm.py:44-56; RMSNorm.forward :16-24 is the SkipIn=None case):
+    s = X + SkipIn in X's dtype; y = float(s) * rsqrt(mean(float(s)^2) + eps);
+    Y = y.type_as(X) * weight (a product in X's dtype); SkipOut = s.  Returns (Y, s)."""
+    s = X if SkipIn is None else X + SkipIn
+    x = s.float()
+    y = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps)
+    return y.to(X.dtype) * weight, s
+
+
+def rms_norm(X, weight, eps=1e-5):
+    """RMSNorm (torch_function/RMSNorm.py:16-24)."""
+    return skip_rms_norm(X, weight, None, eps)[0]
+
+
 def moe_reduce(Y: torch.Tensor, expert_weights: torch.Tensor, invert_permutation: torch.Tensor,
                num_experts_per_token: int, acc=torch.float32, out_dtype=None):
     """``out[t] = sum_s w[t,s] * Y_flat[inv[t,s]]`` summed in slot order."""

@@ -193,6 +193,16 @@ int opmx_silu(const void *X, const void *gate, int64_t n, int dtype, void *Y, vo
     return launch_silu(X, gate, n, dtype, Y, st(stream));
 }
 
+int opmx_rms_norm(const void *X, const void *weight, const void *SkipIn, int64_t T, int64_t H, float eps, int dtype,
+                  void *Y, void *SkipOut, void *stream)
+{
+    if (T < 0 || H < 0) return OPMX_ERR_BAD_ARGUMENT;
+    if (!dtype_ok(dtype)) return OPMX_ERR_UNSUPPORTED;
+    if (T > 0 && H > 0 && (!X || !weight || !Y)) return OPMX_ERR_BAD_ARGUMENT;
+    if (!(eps >= 0.0f)) return OPMX_ERR_BAD_ARGUMENT;
+    return launch_rms_norm(X, weight, SkipIn, T, H, eps, dtype, Y, SkipOut, st(stream));
+}
+
 int opmx_moe_reduce(const void *Y, const void *expert_weights, const int64_t *invert_permutation, int64_t T,
                     int k, int64_t N, int dtype, void *out, void *stream)
 {

@@ -73,6 +73,8 @@ int launch_moe_select(const void *X, const void *scores, int64_t T, int64_t H, i
 size_t moe_select_workspace_bytes(int64_t T, int E, int k);
 int launch_swiglu(const void *X, int64_t R, int64_t D, float beta, int dtype, void *Y, hipStream_t s);
 int launch_silu(const void *X, const void *gate, int64_t n, int dtype, void *Y, hipStream_t s);
+int launch_rms_norm(const void *X, const void *Wt, const void *Skip, int64_t T, int64_t H, float eps, int dtype,
+                    void *Y, void *SkipOut, hipStream_t s);
 int launch_moe_reduce(const void *Y, const void *w, const int64_t *inv, int64_t T, int k, int64_t N,
                       int dtype, void *out, hipStream_t s);
 int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const void *B, int E,

@@ -1,5 +1,6 @@
-"""Router gate module.  Mirrors ``model_zoo/ModelLayers.py:51-69`` of
-OpenPPL/ppl.pmx (weight ``[out_features, in_features]``, optional bias)."""
+"""Router gate module and the norm in front of the MoE layer.  Mirror
+``model_zoo/ModelLayers.py:32-69`` of OpenPPL/ppl.pmx (``RMSNorm``, ``SkipRMSNorm``: weight
+``[dim]`` of ones; ``Linear``: weight ``[out_features, in_features]``, optional bias)."""
 import os
 import sys
 
@@ -8,6 +9,26 @@ from torch import nn
 
 sys.path.append(os.path.join(os.path.dirname(os.path.abspath(__file__)), ".."))
 import torch_function as OPMX  # noqa: E402
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, dim: int, eps: float = 1e-6, dtype=None, device=None):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(dim, dtype=dtype, device=device), requires_grad=False)
+
+    def forward(self, x):
+        return OPMX.rms_norm(x, self.weight, -1, self.eps)
+
+
+class SkipRMSNorm(nn.Module):
+    def __init__(self, dim: int, eps: float = 1e-6, dtype=None, device=None):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(dim, dtype=dtype, device=device), requires_grad=False)
+
+    def forward(self, x, skip):
+        return OPMX.skip_rms_norm(x, self.weight, skip, -1, self.eps)
 
 
 class Linear(nn.Module):

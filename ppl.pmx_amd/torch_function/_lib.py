@@ -38,6 +38,7 @@ _SIGNATURES = {
                                             _vp, _vp, _sz, _vp]),
     "opmx_swiglu": (_int, [_vp, _i64, _i64, _f, _int, _vp, _vp]),
     "opmx_silu": (_int, [_vp, _vp, _i64, _int, _vp, _vp]),
+    "opmx_rms_norm": (_int, [_vp, _vp, _vp, _i64, _i64, _f, _int, _vp, _vp, _vp]),
     "opmx_moe_reduce": (_int, [_vp, _vp, _vp, _i64, _int, _i64, _int, _vp, _vp]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

@@ -62,6 +62,10 @@ def test_argument_validation_needs_no_device(lib):
     assert lib.opmx_swiglu(None, 4, 8, 1.0, 1, one, None) == -1
     assert lib.opmx_silu(one, None, 8, 9, one, None) == -2
     assert lib.opmx_linear(one, one, None, 4, 0, 8, 1, one, None) == -1
+    assert lib.opmx_rms_norm(one, None, None, 4, 8, 1e-5, 1, one, None, None) == -1      # no weight
+    assert lib.opmx_rms_norm(one, one, None, 4, 8, -1.0, 1, one, None, None) == -1       # eps < 0
+    assert lib.opmx_rms_norm(one, one, None, 4, 8, 1e-5, 5, one, None, None) == -2       # dtype
+    assert lib.opmx_rms_norm(None, None, None, 0, 8, 1e-5, 1, None, None, None) == 0     # empty
     # empty problems are no-ops that succeed
     assert lib.opmx_moe_reduce(None, None, None, 0, 2, 8, 1, None, None) == 0
     assert lib.opmx_swiglu(None, 0, 8, 1.0, 1, None, None) == 0

@@ -26,6 +26,9 @@ def test_public_names_and_signatures():
                                                  "in_features", "out_features", "input_is_parallel"]
     assert sig(OPMX.swiglu) == ["X", "beta"] and sig(OPMX.silu) == ["X", "gate"]
     assert sig(OPMX.linear) == ["X", "W", "B", "in_features", "out_features"]
+    assert sig(OPMX.rms_norm) == ["X", "weight", "axis", "eps"]                       # RMSNorm.py:59-61
+    assert sig(OPMX.skip_rms_norm) == ["X", "weight", "SkipIn", "axis", "eps"]        # RMSNorm.py:64-66
+    assert inspect.signature(OPMX.skip_rms_norm).parameters["eps"].default == 1e-5
     p = inspect.signature(OPMX.moe_column_parallel_linear).parameters
     assert p["gather_output"].default is True
     assert inspect.signature(OPMX.moe_row_parallel_linear).parameters["input_is_parallel"].default is False
@@ -41,6 +44,8 @@ def test_no_cpu_fallback():
         OPMX.moe_reduce(torch.randn(4, 2, 8), torch.rand(4, 2), torch.arange(8).view(4, 2), 2)
     with pytest.raises(RuntimeError, match="no CPU path"):
         OPMX.linear(x, torch.randn(8, 16), None, 16, 8)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        OPMX.skip_rms_norm(x, torch.ones(16), x)
     with pytest.raises(AssertionError):          # the reference's in_features assert comes first
         OPMX.moe_column_parallel_linear(x, torch.arange(3), torch.randn(2, 8, 16), None, None, 2, 15, 8, False)
 
@@ -91,6 +96,26 @@ def test_mixtral_block_exports_reference_nodes(fused, bias):
              ("opmx::MoeReduce", 3, 1, dict(num_experts_per_token=k))]
     assert got == want
     assert tuple(out.shape) == (5, H)
+
+
+def test_rms_norm_exports_reference_nodes():
+    """opmx::RMSNorm with axis / eps / skip_term and one or two outputs (RMSNorm.py:6-11, 29-39)."""
+    from model_zoo.ModelLayers import RMSNorm, SkipRMSNorm
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a, self.b = RMSNorm(16, 1e-6), SkipRMSNorm(16, 1e-6)
+
+        def forward(self, x, skip):
+            y, so = self.b(x, skip)
+            return self.a(y), so
+    graph, out = export_graph(Block(), (torch.randn(3, 16), torch.randn(3, 16)))
+    got = nodes_of(graph)
+    assert [(k, i, o) for k, i, o, _ in got] == [("opmx::RMSNorm", 3, 2), ("opmx::RMSNorm", 2, 1)]
+    assert got[0][3]["axis"] == -1 and got[0][3]["skip_term"] == 1 and abs(got[0][3]["eps"] - 1e-6) < 1e-12
+    assert got[1][3]["skip_term"] == 0
+    assert tuple(out[0].shape) == (3, 16) and tuple(out[1].shape) == (3, 16)
 
 
 def test_export_placeholders_have_eager_order_and_types():

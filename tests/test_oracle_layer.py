@@ -126,3 +126,36 @@ def test_make_inputs_is_deterministic():
     b = O.make_inputs(4, 8, 2, 6, seed=0)
     assert all(torch.equal(p, q) for p, q in zip(a, b))
     assert a[2].shape == (2, 12, 8) and a[3].shape == (2, 8, 6)
+
+
+def test_rms_norm_pins():
+    """skip_rms_norm / rms_norm (RMSNorm.py:16-24, 44-56) against a library routine, closed
+    forms and the properties the definition fixes."""
+    g = torch.Generator().manual_seed(5)
+    X = torch.randn(6, 96, generator=g)
+    S = torch.randn(6, 96, generator=g)
+    w = torch.rand(96, generator=g) + 0.5
+    # library routine (independent implementation)
+    assert torch.allclose(O.rms_norm(X, w, 1e-5), F.rms_norm(X, (96,), w, 1e-5), atol=1e-6)
+    Y, so = O.skip_rms_norm(X, w, S, 1e-6)
+    assert torch.equal(so, X + S)                                        # skip output is the plain sum
+    assert torch.allclose(Y, F.rms_norm(X + S, (96,), w, 1e-6), atol=1e-6)
+    # closed forms: a constant row c normalises to sign(c) * weight; weights of one give unit RMS
+    c = torch.full((1, 32), -3.0)
+    assert torch.allclose(O.rms_norm(c, torch.arange(32.0), 0.0), -torch.arange(32.0).view(1, 32))
+    assert torch.allclose(O.rms_norm(X, torch.ones(96), 0.0).pow(2).mean(-1), torch.ones(6), atol=1e-5)
+    # scale invariance without eps, and eps really sits under the root: a zero row stays zero
+    assert torch.allclose(O.rms_norm(7.5 * X, w, 0.0), O.rms_norm(X, w, 0.0), atol=1e-5)
+    assert torch.equal(O.rms_norm(torch.zeros(2, 8), torch.ones(8), 1e-5), torch.zeros(2, 8))
+    row = torch.tensor([[3.0, 4.0]])                                     # mean square 12.5
+    assert torch.allclose(O.rms_norm(row, torch.ones(2), 3.5), row / 4.0)  # sqrt(12.5 + 3.5) = 4
+    # without a skip input the skip output is X itself
+    assert O.skip_rms_norm(X, w)[1] is X
+    # low precision: the sum is rounded to the input dtype before the norm, the normalised value
+    # is rounded before the multiply by the weight (two roundings, as the reference's type_as)
+    Xh, Sh, wh = X.half(), S.half(), w.half()
+    Yh, soh = O.skip_rms_norm(Xh, wh, Sh, 1e-5)
+    assert soh.dtype == torch.float16 and torch.equal(soh, Xh + Sh)
+    x32 = soh.float()
+    y16 = (x32 * torch.rsqrt((x32 * x32).mean(-1, keepdim=True) + 1e-5)).half()
+    assert torch.equal(Yh, (y16.float() * wh.float()).half())
