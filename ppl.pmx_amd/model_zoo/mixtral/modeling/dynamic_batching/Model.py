@@ -4,7 +4,11 @@ Only ``MoeFeedForward`` of the reference's Mixtral model is mirrored here
 (``model_zoo/mixtral/modeling/dynamic_batching/Model.py:155-214`` of
 OpenPPL/ppl.pmx): the six-operator sequence router gate -> MoeSelect ->
 gate/up grouped GEMM -> SwiGLU -> down grouped GEMM -> MoeReduce, with the
-fused weight layout ``wu[e] = [w1[e]; w3[e]]`` of ``Model.py:399-413``.
+fused weight layout ``wu[e] = [w1[e]; w3[e]]`` of ``Model.py:399-413``, and the part
+of ``Transformer.load_state_dict`` (``Model.py:363-420``) that fills it from an OPMX
+checkpoint (``layers.N.feed_forward.{gate,w1,w2,w3}.weight`` with the expert
+weights stacked ``[E, out, in]`` by
+``model_zoo/mixtral/huggingface/ConvertWeightToOpmx.py:98-128``).
 """
 import os
 import sys
@@ -72,3 +76,71 @@ class MoeFeedForward(nn.Module):
             x13 = OPMX.silu(self.w1(x_experts, expert_offset), self.w3(x_experts, expert_offset))
         x_out = self.w2(x13, expert_offset)
         return OPMX.moe_reduce(x_out, expert_weights, invert_permutation, k)
+
+    @torch.no_grad()
+    def load_state_dict(self, state_dict, strict: bool = True, prefix=None):
+        """Fills this block from an OPMX state dict (``Model.py:363-420``).
+
+        Keys are taken under ``prefix`` (default ``layers.<layer_id>.feed_forward.``): ``gate.weight``
+        ``[E,H]``, ``w2.weight`` ``[E,H,I]`` and either ``wu.weight`` ``[E,2I,H]`` or the pair
+        ``w1.weight`` / ``w3.weight`` ``[E,I,H]`` -- with ``fused_ffn_glu`` the pair lands in the two
+        halves of ``wu`` (``Model.py:399-413``); biases likewise.  Tensors are copied into the existing
+        parameters (their dtype and device win), nothing is re-tiled.  Returns the keys it used;
+        ``strict`` raises on a parameter left without a value or a shape mismatch.
+        """
+        prefix = "layers.{}.feed_forward.".format(self.layer_id) if prefix is None else prefix
+        params = dict(self.named_parameters())
+        used, filled = [], set()
+
+        def put(name, value, rows=None):
+            dst = params[name]
+            view = dst if rows is None else dst[:, rows[0]:rows[1]]
+            if tuple(view.shape) != tuple(value.shape):
+                raise ValueError("{}{}: checkpoint has {}, the block expects {}".format(
+                    prefix, name, tuple(value.shape), tuple(view.shape)))
+            view.copy_(value)
+            filled.add((name, rows))
+
+        for key, value in state_dict.items():
+            if not key.startswith(prefix):
+                continue
+            name = key[len(prefix):]
+            module, _, leaf = name.rpartition(".")
+            if name in params:
+                put(name, value)
+            elif self.fused_ffn_glu and module in ("w1", "w3") and "wu." + leaf in params:
+                half = params["wu." + leaf].shape[1] // 2
+                put("wu." + leaf, value, (0, half) if module == "w1" else (half, 2 * half))
+            else:
+                continue
+            used.append(key)
+        if strict:
+            for name in params:
+                whole = (name, None) in filled
+                halves = name.startswith("wu.") and all(
+                    (name, r) in filled for r in ((0, params[name].shape[1] // 2),
+                                                  (params[name].shape[1] // 2, params[name].shape[1])))
+                if not (whole or halves):
+                    raise KeyError("no value for {}{} in the checkpoint".format(prefix, name))
+        return used
+
+
+def load_opmx_moe_block(path, layer_id: int, num_experts_per_token: int, fused_ffn_glu: bool = True,
+                        dtype=None, device=None, fuse_swiglu_epilogue: bool = False):
+    """Builds the MoE block of layer ``layer_id`` from an OPMX Mixtral ``.pth`` checkpoint.
+
+    The file is opened with ``weights_only=True`` and memory-mapped, so only this layer's tensors are
+    read; sizes come from the tensors themselves (``gate.weight`` is ``[E,H]``, ``w2.weight``
+    ``[E,H,I]``).  ``num_experts_per_token`` is not stored in the checkpoint (the reference reads it
+    from ``opmx_params.json``).
+    """
+    sd = torch.load(path, map_location="cpu", weights_only=True, mmap=True)
+    prefix = "layers.{}.feed_forward.".format(layer_id)
+    gate, w2 = sd[prefix + "gate.weight"], sd[prefix + "w2.weight"]
+    E, H = gate.shape
+    bias = (prefix + "w2.bias") in sd
+    block = MoeFeedForward(MoeFeedForward.params(H, w2.shape[2], E, num_experts_per_token), layer_id, fused_ffn_glu,
+                           bias, None, dtype=gate.dtype if dtype is None else dtype, device=device,
+                           fuse_swiglu_epilogue=fuse_swiglu_epilogue)
+    block.load_state_dict(sd)
+    return block

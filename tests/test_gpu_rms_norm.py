@@ -88,3 +88,22 @@ def test_norm_feeds_the_moe_layer():
     assert (y.cpu().float() - yr.float()).abs().max() <= 2e-2
     err = (out.cpu().float() - ref.float()).abs()
     assert err.max() <= 2e-2 and err.mean() <= 2e-3
+
+
+def test_block_from_checkpoint_runs_on_the_gpu(tmp_path):
+    """OPMX checkpoint file -> MoE block on the GPU (stacked expert weights, w1 / w3 into wu)."""
+    from model_zoo.mixtral.modeling.dynamic_batching.Model import load_opmx_moe_block
+    T, H, I, E, k = 40, 256, 384, 8, 2
+    x, Wg, wu, w2 = O.make_inputs(T, H, E, I, dtype=torch.float16, seed=21)
+    p = "layers.3.feed_forward."
+    sd = {p + "gate.weight": Wg, p + "w1.weight": wu[:, :I].contiguous(), p + "w3.weight": wu[:, I:].contiguous(),
+          p + "w2.weight": w2, "layers.3.ffn_norm.weight": torch.ones(H, dtype=torch.float16)}
+    path = tmp_path / "model.pth"
+    torch.save(sd, path)
+    block = load_opmx_moe_block(str(path), 3, k, device=dev())
+    assert block.wu.weight.device.type == "cuda" and torch.equal(block.wu.weight.cpu(), wu)
+    out = block(x.to(dev()))
+    scores = opmx().linear(x.to(dev()), block.gate.weight, None, H, E)
+    ref = O.moe_layer(x, Wg, wu, w2, E, k, scores=scores.cpu(), round_between_ops=False)
+    err = (out.cpu().float() - ref.float()).abs()
+    assert err.max() <= 2e-2 and err.mean() <= 2e-3

@@ -144,3 +144,56 @@ def test_tensor_parallel_is_refused():
         with pytest.raises(NotImplementedError):
             OPMX.moe_column_parallel_linear(torch.randn(4, 16), torch.arange(3), torch.randn(2, 8, 16), None,
                                             FakeGroup(), 2, 16, 8, False)
+
+
+def _fake_checkpoint(E=4, H=16, I=24, layers=2, bias=False, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    sd = {}
+    for n in range(layers):
+        p = "layers.{}.feed_forward.".format(n)
+        sd[p + "gate.weight"] = torch.randn(E, H, generator=g)
+        sd[p + "w1.weight"] = torch.randn(E, I, H, generator=g)
+        sd[p + "w3.weight"] = torch.randn(E, I, H, generator=g)
+        sd[p + "w2.weight"] = torch.randn(E, H, I, generator=g)
+        if bias:
+            sd[p + "w1.bias"] = torch.randn(E, I, generator=g)
+            sd[p + "w3.bias"] = torch.randn(E, I, generator=g)
+            sd[p + "w2.bias"] = torch.randn(E, H, generator=g)
+        sd["layers.{}.ffn_norm.weight".format(n)] = torch.ones(H)
+        sd["layers.{}.attention.wo.weight".format(n)] = torch.randn(H, H, generator=g)
+    return sd
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("bias", [False, True])
+def test_moe_block_loads_an_opmx_checkpoint(tmp_path, fused, bias):
+    """Checkpoint keys and stacked expert layout of ConvertWeightToOpmx.py:98-128; w1 / w3 land in the
+    halves of wu as in Model.py:399-413."""
+    from model_zoo.mixtral.modeling.dynamic_batching.Model import load_opmx_moe_block
+    E, H, I = 4, 16, 24
+    sd = _fake_checkpoint(E, H, I, bias=bias)
+    m = MoeFeedForward(MoeFeedForward.params(H, I, E, 2), 1, fused, bias, None)
+    used = m.load_state_dict(sd)
+    p = "layers.1.feed_forward."
+    assert sorted(used) == sorted(k for k in sd if k.startswith(p))
+    assert torch.equal(m.gate.weight, sd[p + "gate.weight"]) and torch.equal(m.w2.weight, sd[p + "w2.weight"])
+    if fused:
+        assert torch.equal(m.wu.weight[:, :I], sd[p + "w1.weight"]) and torch.equal(m.wu.weight[:, I:], sd[p + "w3.weight"])
+        if bias:
+            assert torch.equal(m.wu.bias[:, :I], sd[p + "w1.bias"]) and torch.equal(m.wu.bias[:, I:], sd[p + "w3.bias"])
+    else:
+        assert torch.equal(m.w1.weight, sd[p + "w1.weight"]) and torch.equal(m.w3.weight, sd[p + "w3.weight"])
+    # strictness: a missing tensor and a wrong shape are refused
+    broken = {k: v for k, v in sd.items() if not k.endswith("1.feed_forward.w3.weight")}
+    with pytest.raises(KeyError):
+        MoeFeedForward(MoeFeedForward.params(H, I, E, 2), 1, fused, bias, None).load_state_dict(broken)
+    wrong = dict(sd)
+    wrong[p + "w2.weight"] = torch.zeros(E, H, I + 1)
+    with pytest.raises(ValueError):
+        MoeFeedForward(MoeFeedForward.params(H, I, E, 2), 1, fused, bias, None).load_state_dict(wrong)
+    # from a file: sizes come from the tensors, dtype can be converted on the way in
+    path = tmp_path / "model.pth"
+    torch.save(sd, path)
+    b = load_opmx_moe_block(str(path), 0, 2, fused_ffn_glu=fused, dtype=torch.float16)
+    assert b.num_experts == E and b.w2.weight.dtype == torch.float16 and (b.w2.bias is not None) == bias
+    assert torch.equal(b.w2.weight, sd["layers.0.feed_forward.w2.weight"].half())
