@@ -51,12 +51,13 @@ __device__ __forceinline__ void stage_offsets(const int64_t *__restrict__ off, i
 // Number of row tiles of height BM over all experts: sum of ceil(rows_e / BM).
 __device__ __forceinline__ int count_mtiles(bool grouped, const int64_t *s_off, int E, int64_t R, int BM)
 {
-    if (!grouped) return static_cast<int>((R + BM - 1) / BM);
+    const int sh = 31 - __builtin_clz(BM);       // BM is a power of two: shifts, not 64-bit divisions
+    if (!grouped) return static_cast<int>((R + BM - 1) >> sh);
     int64_t total = 0, prev = s_off[0];
     for (int e = 0; e < E; ++e) {
         int64_t hi = s_off[e + 1];
         if (hi < prev) hi = prev;
-        total += (hi - prev + BM - 1) / BM;
+        total += (hi - prev + BM - 1) >> sh;
         prev = hi;
     }
     return __builtin_amdgcn_readfirstlane(static_cast<int>(total));
@@ -119,11 +120,12 @@ __device__ __forceinline__ void row_tile(int tile_m, bool grouped, const int64_t
         mt.rows = left <= 0 ? 0 : static_cast<int>(left < BM ? left : BM);
         return;
     }
+    const int sh = 31 - __builtin_clz(BM);       // BM is a power of two
     int64_t tile = tile_m, prev = s_off[0];
     for (int e = 0; e < E; ++e) {
         int64_t hi = s_off[e + 1];
         if (hi < prev) hi = prev;
-        const int64_t nt = (hi - prev + BM - 1) / BM;
+        const int64_t nt = (hi - prev + BM - 1) >> sh;
         if (tile < nt) {
             // block-uniform by construction; say so to the compiler (scalar registers)
             const int64_t row0 = prev + tile * BM, left = hi - row0;
@@ -217,49 +219,93 @@ __device__ __forceinline__ void tile_epilogue(float4_t (&acc)[WTN / 16][WTM / 16
 // bytes instead of 32-byte pieces.  No block barrier is needed (a wave only touches its own
 // region, and its LDS operations execute in order); the caller guarantees that no wave still
 // reads operand tiles from LDS.  Requires ncols % 8 == 0 and a 16-byte aligned Y.
-template <typename T, int WTM, int WTN, bool SWIGLU>
-__device__ __forceinline__ void tile_epilogue_lds(float4_t (&acc)[WTN / 16][WTM / 16], const T *__restrict__ Bias,
-                                                  T *__restrict__ Y, const MTile &mt, int64_t N, int64_t ncols,
-                                                  int64_t n0, int wm, int wn, int lane, char *wave_lds)
+//
+// Everything that does not depend on the sub-tile row i is computed once per lane: the bias of
+// the lane's columns, and the swizzled LDS addresses (a staged row is at most 16 chunks and
+// sub-tiles start at multiples of 16 rows, so row % chunks == (lane % 16) % chunks for every
+// i and the row part of the address is an instruction offset).
+template <typename T, int WTM, int WTN, bool SWIGLU, bool BIAS>
+__device__ __forceinline__ void tile_epilogue_lds_impl(float4_t (&acc)[WTN / 16][WTM / 16], const T *__restrict__ be,
+                                                       T *__restrict__ Y, const MTile &mt, int64_t ncols, int64_t nw0,
+                                                       int wm, int lane, char *wave_lds)
 {
     constexpr int TMS = WTM / 16, TNS = WTN / 16, NO = SWIGLU ? TNS / 2 : TNS;
     constexpr int ROWP = NO * 16 * 2;          // bytes per staged row
     constexpr int CH16 = ROWP / 16;            // 16-byte chunks per staged row
     constexpr int RPI = 1024 / ROWP;           // rows per wave-wide 16-byte access
+    static_assert(16 % CH16 == 0, "a staged row must hold 2, 4, 8 or 16 chunks");
     const int lrow = lane & 15, lk = lane >> 4;
-    const T *be = Bias ? Bias + static_cast<int64_t>(mt.e) * N : nullptr;
-    const int64_t nw0 = (SWIGLU ? n0 + wn * (WTN / 2) : n0 + wn * WTN);   // first output column of this wave
+
+    float bg[BIAS ? NO : 1][4], bu[BIAS && SWIGLU ? NO : 1][4];
+    if (BIAS) {
+#pragma unroll
+        for (int j = 0; j < NO; ++j)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int64_t n = nw0 + j * 16 + lk * 4 + v;
+                const int64_t nn = n < ncols ? n : ncols - 1;
+                bg[j][v] = to_f32(be[nn]);
+                if (SWIGLU) bu[j][v] = to_f32(be[ncols + nn]);
+            }
+    }
+
+    // chunk j*2 + lk/2 of row lrow (+ i*16) lands in slot chunk ^ (lrow % CH16)
+    char *wbase = wave_lds + lrow * ROWP + (lk & 1) * 8;
+    const int c0 = ((lk >> 1) ^ (lrow % CH16)) << 4;
 #pragma unroll
     for (int i = 0; i < TMS; ++i) {
-        const int row = i * 16 + lrow;
 #pragma unroll
         for (int j = 0; j < NO; ++j) {
-            const int64_t n = nw0 + j * 16 + lk * 4;
             T out[4];
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                const int64_t nn = n + v < ncols ? n + v : ncols - 1;
-                float g = acc[j][i][v] + (be ? to_f32(be[nn]) : 0.0f);
+                float g = acc[j][i][v];
+                if (BIAS) g += bg[j][v];
                 if (SWIGLU) {
-                    const float up = acc[j + TNS / 2][i][v] + (be ? to_f32(be[ncols + nn]) : 0.0f);
+                    float up = acc[j + TNS / 2][i][v];
+                    if (BIAS) up += bu[j][v];
                     g = up * g * sigmoid_fast_(g);
                 }
                 out[v] = from_f32<T>(g);
             }
-            const int chunk = j * 2 + (lk >> 1);
-            *reinterpret_cast<uint2 *>(wave_lds + row * ROWP + ((chunk ^ (row % CH16)) << 4) + (lk & 1) * 8) =
-                *reinterpret_cast<const uint2 *>(out);
+            *reinterpret_cast<uint2 *>(wbase + (c0 ^ (j * 32)) + i * 16 * ROWP) = *reinterpret_cast<const uint2 *>(out);
         }
     }
+
+    // read back whole rows: lane reads chunk c of row rr*RPI + lane/CH16
+    const int c = lane % CH16, r0 = lane / CH16;
+    const int64_t n = nw0 + c * 8;
+    const bool col_ok = n < ncols;             // ncols % 8 == 0: a chunk is inside or outside as a whole
+    T *yp = Y + (mt.row0 + wm * WTM + r0) * ncols + n;
+    const int rows_left = static_cast<int>(mt.rows) - wm * WTM - r0;   // row rr*RPI is stored iff rr*RPI < rows_left
+    constexpr int NR = WTM / RPI, BATCH = NR < 8 ? NR : 8;   // LDS reads in flight before their stores
 #pragma unroll
-    for (int rr = 0; rr < WTM / RPI; ++rr) {
-        const int row = rr * RPI + lane / CH16, c = lane % CH16;
-        const u32x4 v = *reinterpret_cast<const u32x4 *>(wave_lds + row * ROWP + ((c ^ (row % CH16)) << 4));
-        const int grow = wm * WTM + row;
-        const int64_t n = nw0 + c * 8;
-        if (grow < mt.rows && n < ncols)       // ncols % 8 == 0: a chunk is inside or outside as a whole
-            *reinterpret_cast<u32x4 *>(Y + (mt.row0 + grow) * ncols + n) = v;
+    for (int r8 = 0; r8 < NR; r8 += BATCH) {
+        u32x4 v[BATCH];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+            const int row = (r8 + u) * RPI + r0;   // row % CH16 takes CH16 / RPI (1 or 4) distinct per-lane values
+            v[u] = *reinterpret_cast<const u32x4 *>(wave_lds + row * ROWP + ((c ^ (row % CH16)) << 4));
+        }
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+            if (col_ok && (r8 + u) * RPI < rows_left) *reinterpret_cast<u32x4 *>(yp) = v[u];
+            yp += static_cast<int64_t>(RPI) * ncols;
+        }
     }
+}
+
+template <typename T, int WTM, int WTN, bool SWIGLU>
+__device__ __forceinline__ void tile_epilogue_lds(float4_t (&acc)[WTN / 16][WTM / 16], const T *__restrict__ Bias,
+                                                  T *__restrict__ Y, const MTile &mt, int64_t N, int64_t ncols,
+                                                  int64_t n0, int wm, int wn, int lane, char *wave_lds)
+{
+    const int64_t nw0 = (SWIGLU ? n0 + wn * (WTN / 2) : n0 + wn * WTN);   // first output column of this wave
+    if (Bias)
+        tile_epilogue_lds_impl<T, WTM, WTN, SWIGLU, true>(acc, Bias + static_cast<int64_t>(mt.e) * N, Y, mt, ncols, nw0,
+                                                          wm, lane, wave_lds);
+    else
+        tile_epilogue_lds_impl<T, WTM, WTN, SWIGLU, false>(acc, nullptr, Y, mt, ncols, nw0, wm, lane, wave_lds);
 }
 
 // Register-staged kernel: two LDS buffers, ONE register set staging global -> LDS, one barrier
@@ -483,9 +529,15 @@ __device__ __forceinline__ void barrier_no_fence()
 
 // Raw buffer descriptor over [base, base + 4 GiB): loads through it take a scalar base, a
 // scalar offset and a 32-bit lane offset.
+// `base` must be the same in every lane: it is forced into scalar registers, because a
+// descriptor the compiler cannot prove uniform turns every load into a loop over lanes.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t raw_descriptor(const void *base)
 {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, static_cast<int>(0xFFFFFFFFu), 0x00020000);
+    const uint64_t b = reinterpret_cast<uint64_t>(base);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(b));
+    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(b >> 32));
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>((static_cast<uint64_t>(hi) << 32) | lo), 0,
+                                             static_cast<int>(0xFFFFFFFFu), 0x00020000);
 }
 
 // 16 bytes per lane from descriptor + soff + voff straight into LDS at lds + 16*lane (lds is
@@ -741,8 +793,15 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
 #undef OPMX_XFRAG
 #undef OPMX_ISSUE1
 
-    // asm MFMAs are opaque to the compiler's hazard padding: let the last ones retire
+    // asm MFMAs are opaque to the compiler's hazard padding: let the last ones retire.  The
+    // empty statements re-define every accumulator after the wait, so that whatever the register
+    // allocator does with a finished accumulator (copy it out, spill it) is placed behind the
+    // wait and not directly behind the MFMA that produced it, where it would read stale data.
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+    for (int j = 0; j < TNS; ++j)
+#pragma unroll
+        for (int i = 0; i < TMS; ++i) asm volatile("" : "+a"(acc[j][i]));
 
     if (SK) {
         // A k-range of a tail tile.  Every workgroup parks its fp32 partial sums in its own slot
