@@ -33,6 +33,13 @@ template <> struct Mfma<f16> {
     {
         asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
+    // c = a*b (addend 0) into an accumulation register quad: starts a new accumulation without
+    // clearing the accumulators, and without carrying their old values along (in a loop over
+    // tiles that would make them loop-carried values the register allocator moves about).
+    static __device__ __forceinline__ void m16_first(frag a, frag b, float4_t &c)
+    {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
+    }
 };
 template <> struct Mfma<bf16> {
     using frag = bf16x8_t;
@@ -47,6 +54,13 @@ template <> struct Mfma<bf16> {
     static __device__ __forceinline__ void m16_acc(frag a, frag b, float4_t &c)
     {
         asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
+    // c = a*b (addend 0) into an accumulation register quad: starts a new accumulation without
+    // clearing the accumulators, and without carrying their old values along (in a loop over
+    // tiles that would make them loop-carried values the register allocator moves about).
+    static __device__ __forceinline__ void m16_first(frag a, frag b, float4_t &c)
+    {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
     }
 };
 

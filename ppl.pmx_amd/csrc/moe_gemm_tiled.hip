@@ -527,6 +527,17 @@ __device__ __forceinline__ void barrier_no_fence()
     asm volatile("" ::: "memory");
 }
 
+// Waits until at most N vector-memory operations of this wave are outstanding (they complete
+// in issue order, loads and stores alike).
+template <int N> __device__ __forceinline__ void wait_vm()
+{
+    static_assert(N == 0 || N == 16 || N == 32 || N == 48, "add the immediate here");
+    if (N == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (N == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    if (N == 32) asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
+    if (N == 48) asm volatile("s_waitcnt vmcnt(48)" ::: "memory");
+}
+
 // Raw buffer descriptor over [base, base + 4 GiB): loads through it take a scalar base, a
 // scalar offset and a 32-bit lane offset.
 // `base` must be the same in every lane: it is forced into scalar registers, because a
@@ -545,6 +556,41 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t raw_descriptor(const void *bas
 __device__ __forceinline__ void load_to_lds_16(__amdgpu_buffer_rsrc_t r, char *lds, uint32_t voff, int soff)
 {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(r, OPMX_LPTR(lds), 16, voff, soff, 0, 0);
+}
+
+// This lane's share of the sixteen 1 KiB wave loads per operand and k-tile: load i of wave w
+// fetches tile rows 8*(w*L+i) .. +7, lane l the 16-byte chunk of row 8*(w*L+i) + l/8 that
+// belongs in LDS slot l%8 of that row (slots are XOR-swizzled by row).  Results are byte offsets
+// from the tile's X rows / the expert's W at k = 0; rows past the tile or the matrix repeat the
+// last valid row (they feed accumulators that are never stored).  With SWIGLU a wave's WTN
+// W-rows are WTN/2 gate rows followed by the WTN/2 up rows of the same output columns.
+template <int LA, int LB, int WTN, bool SWIGLU>
+__device__ __forceinline__ void tile_sources(int rows, int64_t n0, int64_t K, int64_t N, int64_t ncols, int wave,
+                                             int lane, uint32_t (&a_src)[LA], uint32_t (&b_src)[LB])
+{
+    const int lrow8 = lane >> 3, slot = lane & 7;
+#pragma unroll
+    for (int i = 0; i < LA; ++i) {
+        const int row = (wave * LA + i) * 8 + lrow8;
+        const int r = row < rows ? row : rows - 1;
+        const int c = slot ^ ((row >> 1) & 7);
+        a_src[i] = static_cast<uint32_t>((r * K + c * 8) * 2);
+    }
+#pragma unroll
+    for (int i = 0; i < LB; ++i) {
+        const int row = (wave * LB + i) * 8 + lrow8;
+        int64_t wrow;
+        if (SWIGLU) {
+            const int w = row / WTN, jj = row % WTN, half = jj / (WTN / 2);
+            int64_t ii = n0 + w * (WTN / 2) + jj % (WTN / 2);
+            ii = ii < ncols ? ii : ncols - 1;
+            wrow = half * ncols + ii;
+        } else {
+            wrow = n0 + row < N ? n0 + row : N - 1;
+        }
+        const int c = slot ^ ((row >> 1) & 7);
+        b_src[i] = static_cast<uint32_t>((wrow * K + c * 8) * 2);
+    }
 }
 
 // Tail balancing ("split-K of the last round").  With G workgroup slots (one per CU) the last
@@ -673,31 +719,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
     const __amdgpu_buffer_rsrc_t rx = raw_descriptor(X + mt.row0 * K);
     const __amdgpu_buffer_rsrc_t rw = raw_descriptor(W + static_cast<int64_t>(mt.e) * N * K);
 
-    // this lane's share of the wave loads: tile row 8*(wave*L+i) + lane/8, LDS slot lane%8
-    const int lrow8 = lane >> 3, slot = lane & 7;
     uint32_t a_src[LA], b_src[LB];     // byte offsets from the tile's X / W base at k = 0
-#pragma unroll
-    for (int i = 0; i < LA; ++i) {
-        const int row = (wave * LA + i) * 8 + lrow8;
-        const int r = row < mt.rows ? row : mt.rows - 1;
-        const int c = slot ^ ((row >> 1) & 7);
-        a_src[i] = static_cast<uint32_t>((r * K + c * 8) * 2);
-    }
-#pragma unroll
-    for (int i = 0; i < LB; ++i) {
-        const int row = (wave * LB + i) * 8 + lrow8;
-        int64_t wrow;
-        if (SWIGLU) {
-            const int w = row / WTN, jj = row % WTN, half = jj / (WTN / 2);
-            int64_t ii = n0 + w * (WTN / 2) + jj % (WTN / 2);
-            ii = ii < ncols ? ii : ncols - 1;
-            wrow = half * ncols + ii;
-        } else {
-            wrow = n0 + row < N ? n0 + row : N - 1;
-        }
-        const int c = slot ^ ((row >> 1) & 7);
-        b_src[i] = static_cast<uint32_t>((wrow * K + c * 8) * 2);
-    }
+    tile_sources<LA, LB, WTN, SWIGLU>(mt.rows, n0, K, N, ncols, wave, lane, a_src, b_src);
     const int a_lds = wave * LA * 1024, b_lds = BM * ROWB + wave * LB * 1024;   // wave-uniform
 
     float4_t acc[TNS][TMS];
@@ -728,11 +751,20 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
 #define OPMX_WFRAG(BUF, S, J)                                                                      \
     wf[S][J] = *reinterpret_cast<const frag *>(smem + (BUF)*STAGE + ((S) ? co1 : co0) + w_off + (J)*16 * ROWB)
 #define OPMX_MF(S, H, m) Mfma<T>::m16_acc(wf[S][(m) % TNS], xf[S][H][(m) / TNS], acc[(m) % TNS][(H)*HM + (m) / TNS])
-    // k-tile in buffer B.  LD2: k-tile KT+2 exists (loaded into buffer B).  NEXT: k-tile KT+1 exists.
-#define OPMX_ITER(KT, B, LD2, NEXT)                                                                \
+    // the first k-tile of a tile overwrites the accumulators instead of adding to them
+#define OPMX_MF0(FIRST, H, m)                                                                      \
+    do {                                                                                           \
+        if (FIRST) Mfma<T>::m16_first(wf[0][(m) % TNS], xf[0][H][(m) / TNS], acc[(m) % TNS][(H)*HM + (m) / TNS]); \
+        else OPMX_MF(0, H, m);                                                                     \
+    } while (0)
+    // One k-tile, held in buffer B.  LD2: load k-tile LDK (of this tile: two k-tiles ahead; or one
+    // of the first two of the workgroup's next tile) into buffer B once it is free, then wait
+    // until at most VM vector-memory operations are outstanding; without LD2 wait for all.
+    // NEXT: read the first fragments of the following k-tile from the other buffer.
+#define OPMX_ITERX(LDK, B, LD2, NEXT, FIRST, VM)                                                   \
     do {                                                                                           \
         _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
-            OPMX_MF(0, 0, m);                                                                      \
+            OPMX_MF0(FIRST, 0, m);                                                                 \
             if (m % 2 == 0) {                                                                      \
                 const int r = m / 2;                                                               \
                 if (r < 4) OPMX_XFRAG(B, 0, 1, r < 4 ? r : 0);                                     \
@@ -741,17 +773,16 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
             }                                                                                      \
         }                                                                                          \
         _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
-            OPMX_MF(0, 1, m);                                                                      \
+            OPMX_MF0(FIRST, 1, m);                                                                 \
             if (m < 4) OPMX_XFRAG(B, 1, 1, m < 4 ? m : 0);                                         \
             if (m == 10) barrier_no_fence();                                                       \
-            if ((LD2) && m >= 11 && (m - 11) % 3 == 0) OPMX_ISSUE1((KT) + 2, B, (m - 11) / 3);     \
+            if ((LD2) && m >= 11 && (m - 11) % 3 == 0) OPMX_ISSUE1(LDK, B, (m - 11) / 3);          \
         }                                                                                          \
         _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
             OPMX_MF(1, 0, m);                                                                      \
-            if ((LD2) && m % 3 == 0 && m / 3 < 9) OPMX_ISSUE1((KT) + 2, B, 7 + m / 3);             \
+            if ((LD2) && m % 3 == 0 && m / 3 < 9) OPMX_ISSUE1(LDK, B, 7 + m / 3);                  \
         }                                                                                          \
-        if (LD2) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");                                 \
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                      \
+        wait_vm<(LD2) ? (VM) : 0>();                                                               \
         __builtin_amdgcn_s_barrier();                                                              \
         asm volatile("" ::: "memory");                                                             \
         _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
@@ -760,6 +791,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
             else if ((NEXT) && m < 12) OPMX_WFRAG((B) ^ 1, 0, (m >= 4 && m < 12) ? m - 4 : 0);     \
         }                                                                                          \
     } while (0)
+#define OPMX_ITER(KT, B, LD2, NEXT) OPMX_ITERX((KT) + 2, B, LD2, NEXT, false, 16)
 
     // prologue: first k-tile -> buffer 0, second -> buffer 1, wait for the first
 #pragma unroll
@@ -787,12 +819,6 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
         }
         OPMX_ITER(kt, b, false, false);
     }
-#undef OPMX_ITER
-#undef OPMX_MF
-#undef OPMX_WFRAG
-#undef OPMX_XFRAG
-#undef OPMX_ISSUE1
-
     // asm MFMAs are opaque to the compiler's hazard padding: let the last ones retire.  The
     // empty statements re-define every accumulator after the wait, so that whatever the register
     // allocator does with a finished accumulator (copy it out, spill it) is placed behind the
@@ -847,6 +873,284 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
     else
         tile_epilogue<T, WTM, WTN, SWIGLU>(acc, Bias, Y, mt, N, ncols, n0, wm, wn, lane);
 }
+
+// Descriptor over `bytes` bytes from `base` (both uniform): accesses at offsets >= bytes are
+// dropped by the hardware range check.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t bounded_descriptor(const void *base, uint32_t bytes)
+{
+    const uint64_t b = reinterpret_cast<uint64_t>(base);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(b));
+    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(b >> 32));
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>((static_cast<uint64_t>(hi) << 32) | lo), 0,
+                                             static_cast<int>(__builtin_amdgcn_readfirstlane(bytes)), 0x00020000);
+}
+__device__ __forceinline__ void store_16(__amdgpu_buffer_rsrc_t r, uint32_t voff, u32x4 v)
+{
+    __builtin_amdgcn_raw_buffer_store_b128(v, r, voff, 0, 0);
+}
+constexpr uint32_t kDroppedStore = 0x80000000u;   // an offset past every tile (tiles are < 2 GiB)
+
+// 8-byte LDS store the compiler does not see as one.  In front of a visible LDS store it waits
+// for every outstanding direct-to-LDS load (it cannot tell that they land elsewhere), which in
+// the persistent kernel are the next tile's first k-tiles, still in flight by design.
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void lds_store_8_untracked(char *p, u32x2 v)
+{
+    const uint32_t a = (uint32_t)(size_t)OPMX_LPTR(p);
+    asm volatile("ds_write_b64 %0, %1" ::"v"(a), "v"(v) : "memory");
+}
+
+// Epilogue of the persistent kernel.  Same values as tile_epilogue_lds, but
+//  - staged through a small wave-private LDS region, 16 rows (one row of sub-tiles) at a time,
+//    because the operand buffers already receive the next tile;
+//  - stored through a descriptor over the tile's rows: lanes outside the tile (rows past its
+//    end, columns past the matrix) get an offset the range check drops, so every wave issues
+//    the same WTM * ROWP / 1024 stores whatever the tile's shape -- the caller's count of
+//    outstanding memory operations depends on that;
+//  - the stores of one pass are issued behind the LDS reads of the next.
+// `ry` covers rows [row0, row0 + rows) of Y; requires ncols % 8 == 0 and a 16-byte aligned Y.
+// The bias of this lane's output columns (gate columns in bg, up columns in bu), for
+// tile_epilogue_staged_impl.  A function of its own so that the persistent kernel can issue
+// these loads ahead of the last loads of a tile: waiting for them in the epilogue then leaves
+// the younger loads of the next tile in flight.
+template <typename T, int NO, bool SWIGLU>
+__device__ __forceinline__ void load_bias_regs(const T *__restrict__ be, int64_t ncols, int64_t nw0, int lane,
+                                               T (&bg)[NO][4], T (&bu)[NO][4])
+{
+    const int lk = lane >> 4;
+#pragma unroll
+    for (int j = 0; j < NO; ++j)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int64_t n = nw0 + j * 16 + lk * 4 + v;
+            const int64_t nn = n < ncols ? n : ncols - 1;
+            bg[j][v] = be[nn];             // left as loaded: converting here would wait for the load here
+            bu[j][v] = be[SWIGLU ? ncols + nn : nn];
+        }
+}
+
+template <typename T, int WTM, int WTN, bool SWIGLU, bool BIAS>
+__device__ __forceinline__ void tile_epilogue_staged_impl(
+    float4_t (&acc)[WTN / 16][WTM / 16], const T (&bg)[SWIGLU ? WTN / 32 : WTN / 16][4],
+    const T (&bu)[SWIGLU ? WTN / 32 : WTN / 16][4], __amdgpu_buffer_rsrc_t ry, int64_t ncols, int64_t nw0, int wm,
+    int lane, char *stg)
+{
+    constexpr int TMS = WTM / 16, TNS = WTN / 16, NO = SWIGLU ? TNS / 2 : TNS;
+    constexpr int ROWP = NO * 16 * 2;          // bytes per staged row
+    constexpr int CH16 = ROWP / 16;            // 16-byte chunks per staged row
+    constexpr int RPI = 1024 / ROWP;           // rows per wave-wide 16-byte access
+    constexpr int NRD = 16 / RPI;              // accesses per pass of 16 rows
+    static_assert(16 % CH16 == 0 && 16 % RPI == 0, "staged row must hold 4, 8 or 16 chunks");
+    const int lrow = lane & 15, lk = lane >> 4;
+    char *wbase = stg + lrow * ROWP + (lk & 1) * 8;
+    const int c0 = ((lk >> 1) ^ (lrow % CH16)) << 4;
+    const int c = lane % CH16, r0 = lane / CH16;
+    const int64_t n = nw0 + c * 8;
+    // byte offset of (tile row wm*WTM + r0, column n); one pass further down is 16 rows
+    uint32_t voff = n < ncols ? static_cast<uint32_t>(((wm * WTM + r0) * ncols + n) * 2) : kDroppedStore;
+    const uint32_t row_bytes = static_cast<uint32_t>(ncols * 2);
+    u32x4 held[NRD];
+#pragma unroll
+    for (int i = 0; i <= TMS; ++i) {
+        // keep every pass's accumulator reads inside the pass: moved to the front they would need
+        // a vector register each while the next tile's fragments and offsets are live
+        __builtin_amdgcn_sched_barrier(0);
+        u32x4 now[NRD];
+        if (i < TMS) {
+#pragma unroll
+            for (int j = 0; j < NO; ++j) {
+                T out[4];
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    float g = acc[j][i][v];
+                    if (BIAS) g += to_f32(bg[j][v]);
+                    if (SWIGLU) {
+                        float up = acc[j + TNS / 2][i][v];
+                        if (BIAS) up += to_f32(bu[j][v]);
+                        g = up * g * sigmoid_fast_(g);
+                    }
+                    out[v] = from_f32<T>(g);
+                }
+                u32x2 bits;
+                __builtin_memcpy(&bits, out, 8);
+                lds_store_8_untracked(wbase + (c0 ^ (j * 32)), bits);
+            }
+#pragma unroll
+            for (int u = 0; u < NRD; ++u) {
+                const int row = u * RPI + r0;
+                now[u] = *reinterpret_cast<const u32x4 *>(stg + row * ROWP + ((c ^ (row % CH16)) << 4));
+            }
+        }
+        if (i > 0) {
+#pragma unroll
+            for (int u = 0; u < NRD; ++u) {
+                // n >= ncols keeps the dropped offset: adding rows to it stays far past the tile
+                store_16(ry, voff, held[u]);
+                voff += (n < ncols ? RPI : 0) * row_bytes;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < NRD; ++u) held[u] = now[u];
+    }
+}
+
+// Persistent form of gemm_tiled_dlds_kernel: one workgroup per CU walks the tile ids
+// blockIdx.x, blockIdx.x + gridDim.x, ... (2-D tile order only, K >= 4 k-tiles) and treats them
+// as one continuous stream of k-tiles.  The last two k-tile steps of a tile already load the
+// first two k-tiles of the next one, so there is no pipeline refill between tiles, and the
+// output stores of a tile drain behind the MFMAs of the next: they are issued after those loads,
+// and vector-memory operations complete in issue order, so the first step of the next tile
+// waits with a count that leaves the stores (a fixed number per wave, see
+// tile_epilogue_staged_impl) and its own new loads outstanding.
+// Covers the tile ids the tail launch does not take (see sk_split).
+template <typename T, int BM, int BN, bool SWIGLU, bool BIAS>
+__global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *__restrict__ X,
+                                                                       const int64_t *__restrict__ off,
+                                                                       const T *__restrict__ W,
+                                                                       const T *__restrict__ Bias, int E, int64_t R,
+                                                                       int64_t K, int64_t N, T *__restrict__ Y,
+                                                                       int ntiles_n, int gnx, int sk_wgs, int sk_cost)
+{
+    constexpr int WM = 2, WN = 2, NW = 4;
+    constexpr int WTM = BM / WM, WTN = BN / WN, TMS = WTM / 16, TNS = WTN / 16, HM = TMS / 2;
+    constexpr int BNO = SWIGLU ? BN / 2 : BN;
+    constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW, NL = LA + LB;
+    constexpr int STAGE = (BM + BN) * ROWB;
+    constexpr int NM = HM * TNS;
+    constexpr int STG = 16 * (SWIGLU ? WTN / 2 : WTN) * 2;            // staging bytes per wave: 16 output rows
+    constexpr int NS = WTM * (SWIGLU ? WTN / 2 : WTN) * 2 / 1024;      // output stores per wave and tile
+    static_assert(HM == 4 && TNS == 8 && NL == 16, "the schedule is written for 128x128 wave tiles");
+    constexpr int NOB = SWIGLU ? TNS / 2 : TNS;                       // output sub-tile columns per wave
+    static_assert(NS == 16 || NS == 32, "wait counts below");
+    using frag = typename Mfma<T>::frag;
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];      // two stages, then NW staging regions
+    __shared__ int64_t s_off[OPMX_MOE_MAX_EXPERTS + 1];
+
+    const int64_t ncols = SWIGLU ? N / 2 : N;
+    zero_unowned_rows(Y, R, ncols, off, E);
+    stage_offsets(off, E, R, s_off);
+    const int mtiles = count_mtiles(off != nullptr, s_off, E, R, BM);
+    const int nk = static_cast<int>(K / BK);
+    const int64_t ttot = static_cast<int64_t>(mtiles) * ntiles_n;
+    const int g = sk_split(ttot, sk_wgs, nk, gnx, sk_cost);
+    const int64_t nmain = g > 1 ? ttot - ttot % sk_wgs : ttot;        // ids [nmain, ttot) are the tail launch's
+    int64_t id = blockIdx.x;
+    if (id >= nmain) return;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    MTile cur;
+    int cur_n;
+    {
+        int tile_m;
+        map_tile(static_cast<int>(id), gnx, mtiles, ntiles_n, tile_m, cur_n);
+        row_tile(tile_m, off != nullptr, s_off, E, R, BM, cur);
+    }
+    if (cur.rows == 0) return;
+    __amdgpu_buffer_rsrc_t rx = raw_descriptor(X + cur.row0 * K);
+    __amdgpu_buffer_rsrc_t rw = raw_descriptor(W + static_cast<int64_t>(cur.e) * N * K);
+    uint32_t a_src[LA], b_src[LB];
+    tile_sources<LA, LB, WTN, SWIGLU>(cur.rows, static_cast<int64_t>(cur_n) * BNO, K, N, ncols, wave, lane, a_src, b_src);
+    const int a_lds = wave * LA * 1024, b_lds = BM * ROWB + wave * LB * 1024;
+    char *stg = smem + 2 * STAGE + wave * STG;
+
+    float4_t acc[TNS][TMS];            // every tile's first k-tile defines all of them
+
+    const int lrow = lane & 15, lk = lane >> 4;
+    const int swz = (lrow >> 1) & 7;
+    const int x_off = (wm * WTM + lrow) * ROWB;
+    const int w_off = BM * ROWB + (wn * WTN + lrow) * ROWB;
+    const int co0 = ((lk ^ swz) << 4), co1 = (((4 + lk) ^ swz) << 4);
+    frag xf[2][2][HM], wf[2][TNS];
+
+#pragma unroll
+    for (int q = 0; q < NL; ++q) OPMX_ISSUE1(0, 0, q);
+#pragma unroll
+    for (int q = 0; q < NL; ++q) OPMX_ISSUE1(1, 1, q);
+    wait_vm<16>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < HM; ++i) OPMX_XFRAG(0, 0, 0, i);
+#pragma unroll
+    for (int j = 0; j < TNS; ++j) OPMX_WFRAG(0, 0, j);
+
+    // The first step of a tile waits with a count that leaves the previous tile's NS stores
+    // outstanding (below).  Give the first tile the same history: NS stores the range check drops.
+    {
+        const __amdgpu_buffer_rsrc_t nowhere = bounded_descriptor(Y, 0);
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int u = 0; u < NS; ++u) store_16(nowhere, kDroppedStore + 16 * u, zero);   // distinct: none is redundant
+    }
+
+    int b = 0;
+    for (;;) {
+        // The workgroup's next tile (uniform).  Without one the last two steps load this tile's
+        // first k-tiles again, into buffers nobody reads any more: one code path for the
+        // accumulators, no matter whether a tile follows.
+        const int64_t nid = id + gridDim.x;
+        MTile nxt = cur;
+        int nxt_n = cur_n;
+        bool has_next = false;
+        if (nid < nmain) {
+            int tile_m;
+            MTile t;
+            map_tile(static_cast<int>(nid), gnx, mtiles, ntiles_n, tile_m, nxt_n);
+            row_tile(tile_m, off != nullptr, s_off, E, R, BM, t);
+            has_next = t.rows > 0;
+            if (has_next) nxt = t;
+            else nxt_n = cur_n;
+        }
+
+        // k-tile 0 overwrites the accumulators.  When k-tile 1 is known to have landed, the NS
+        // stores of the previous tile and the 16 loads of this step may still be outstanding.
+        OPMX_ITERX(2, b, true, true, true, 16 + NS);
+        b ^= 1;
+        for (int kt = 1; kt + 2 < nk; ++kt, b ^= 1) OPMX_ITERX(kt + 2, b, true, true, false, 16);
+        // all loads of this tile are issued: retarget the load state, then stream on
+        rx = raw_descriptor(X + nxt.row0 * K);
+        rw = raw_descriptor(W + static_cast<int64_t>(nxt.e) * N * K);
+        tile_sources<LA, LB, WTN, SWIGLU>(nxt.rows, static_cast<int64_t>(nxt_n) * BNO, K, N, ncols, wave, lane, a_src, b_src);
+        const int64_t nw0 = static_cast<int64_t>(cur_n) * BNO + wn * (SWIGLU ? WTN / 2 : WTN);   // first output column of this wave
+        T bg[NOB][4], bu[NOB][4];          // bias of this lane's columns, requested ahead of the last loads
+        if (BIAS) load_bias_regs<T, NOB, SWIGLU>(Bias + static_cast<int64_t>(cur.e) * N, ncols, nw0, lane, bg, bu);
+        OPMX_ITERX(0, b, true, true, false, 16);
+        b ^= 1;
+        OPMX_ITERX(1, b, true, true, false, 16);
+        b ^= 1;
+        // let the last MFMAs retire; re-define the accumulators behind the wait (see
+        // gemm_tiled_dlds_kernel)
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+        for (int j = 0; j < TNS; ++j)
+#pragma unroll
+            for (int i = 0; i < TMS; ++i) asm volatile("" : "+a"(acc[j][i]));
+
+        {
+            const __amdgpu_buffer_rsrc_t ry =
+                bounded_descriptor(Y + cur.row0 * ncols, static_cast<uint32_t>(cur.rows * ncols * 2));
+            // BIAS is a kernel parameter, not a branch: the bias instance needs registers for the
+            // lane's bias values, and in one kernel the other path would pay for them with spills
+            tile_epilogue_staged_impl<T, WTM, WTN, SWIGLU, BIAS>(acc, bg, bu, ry, ncols, nw0, wm, lane, stg);
+        }
+        if (!has_next) break;
+        cur = nxt;
+        cur_n = nxt_n;
+        id = nid;
+    }
+    // the loads issued for a tile that does not follow must land before the LDS goes away
+    wait_vm<0>();
+}
+#undef OPMX_ITER
+#undef OPMX_ITERX
+#undef OPMX_MF0
+#undef OPMX_MF
+#undef OPMX_WFRAG
+#undef OPMX_XFRAG
+#undef OPMX_ISSUE1
 
 // Clears the arrival counters of the tail tiles (a kernel, not a memset: callers may capture
 // the launch sequence in a graph).
@@ -962,6 +1266,43 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
     }
     const T *Xp = static_cast<const T *>(X), *Wp = static_cast<const T *>(W), *Bp = static_cast<const T *>(B);
     T *Yp = static_cast<T *>(Y);
+    // Persistent form (one workgroup per CU streams through its tiles) whenever its conditions
+    // hold: 2-D tile order, at least 4 k-tiles, whole 16-byte output chunks, tiles under 2 GiB.
+    bool persist = gnx == 4 && K / BK >= 4 && ncols % 8 == 0 && reinterpret_cast<uintptr_t>(Y) % 16 == 0 &&
+                   ncols * (2 * BM) < (int64_t{1} << 31) && cus >= 8 && cus % 8 == 0;
+    if (const char *v = std::getenv("OPMX_MOE_GEMM_PERSIST")) persist = persist && std::atoi(v) != 0;   // tuning knob
+    if (persist) {
+        const int smem_p = smem + 4 * 16 * (sw ? BN / 4 : BN / 2) * 2;       // + the four staging regions
+        static bool attr_p[4] = {false, false, false, false};
+        const bool hb = B != nullptr;
+        using kernel_t = void (*)(const T *, const int64_t *, const T *, const T *, int, int64_t, int64_t, int64_t, T *, int,
+                                  int, int, int);
+        const kernel_t kp = sw ? (hb ? gemm_tiled_dlds_persist_kernel<T, BM, BN, true, true>
+                                     : gemm_tiled_dlds_persist_kernel<T, BM, BN, true, false>)
+                               : (hb ? gemm_tiled_dlds_persist_kernel<T, BM, BN, false, true>
+                                     : gemm_tiled_dlds_persist_kernel<T, BM, BN, false, false>);
+        const int slot = (sw ? 2 : 0) + (hb ? 1 : 0);
+        if (!attr_p[slot]) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kp), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    smem_p) != hipSuccess)
+                return OPMX_ERR_LAUNCH;
+            attr_p[slot] = true;
+        }
+        // ids congruent mod 8 stay on one XCD as long as the grid is a multiple of 8
+        const unsigned wgs = static_cast<unsigned>(dp_ids < cus ? dp_ids : cus);
+        if (sk_wgs > 0) sk_clear_kernel<<<1, 256, 0, s>>>(sk_count, kSkCounters);
+        kp<<<wgs, block, smem_p, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n, gnx, sk_wgs, sk_cost);
+        if (sk_wgs > 0) {
+            if (sw)
+                gemm_tiled_dlds_kernel<T, BM, BN, true, true><<<sk_wgs, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
+                                                                                          gnx, sk_wgs, sk_cost, sk_part, sk_count);
+            else
+                gemm_tiled_dlds_kernel<T, BM, BN, false, true><<<sk_wgs, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
+                                                                                           gnx, sk_wgs, sk_cost, sk_part, sk_count);
+        }
+        OPMX_LAUNCH_CHECK();
+        return OPMX_OK;
+    }
     if (sk_wgs > 0) sk_clear_kernel<<<1, 256, 0, s>>>(sk_count, kSkCounters);
     if (sw) {
         gemm_tiled_dlds_kernel<T, BM, BN, true, false><<<grid, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,

@@ -107,6 +107,23 @@ def test_tile_order_with_partial_last_round(variant):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_persistent_kernel_streams_tiles(dtype):
+    """The persistent form of the 256x256 kernel (16 column tiles, K >= 256): fewer tiles than
+    workgroups, then 27 row tiles x 16 = 432 tiles so that workgroups walk on to a second tile
+    (ragged row tiles, bias, SwiGLU with 16 column tiles of 128), K = 256 being the shortest
+    stream it takes; the one-tile-per-workgroup form must give the same bits."""
+    env = {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": "0", "OPMX_MOE_GEMM_STREAMK": "0"}
+    sizes = [1500, 0, 700, 33, 1281, 256, 5, 1300, 1024, 300]
+    run_case("column", [300, 77, 129], 256, 4096, dtype, True, env)
+    for K, bias, swiglu in ((256, False, False), (320, True, False), (512, True, True), (1024, False, True)):
+        a = run_case("column", sizes, K, 4096, dtype, bias, env, swiglu=swiglu)
+        b = run_case("column", sizes, K, 4096, dtype, bias, dict(env, OPMX_MOE_GEMM_PERSIST="0"), swiglu=swiglu)
+        assert torch.equal(a, b)
+    # with the tail of the last round split over k by the second launch
+    run_case("row", sizes, 1024, 4096, dtype, True, dict(env, OPMX_MOE_GEMM_STREAMK="2"))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_tail_tiles_split_over_k(dtype):
     """Few tiles (4 row tiles x 16 column tiles, 2-D tile order) and a long K: the tail launch of
     the 256x256 kernel cuts every tile into k-ranges whose fp32 partial sums meet in the workspace
