@@ -1266,11 +1266,18 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
     }
     const T *Xp = static_cast<const T *>(X), *Wp = static_cast<const T *>(W), *Bp = static_cast<const T *>(B);
     T *Yp = static_cast<T *>(Y);
-    // Persistent form (one workgroup per CU streams through its tiles) whenever its conditions
-    // hold: 2-D tile order, at least 4 k-tiles, whole 16-byte output chunks, tiles under 2 GiB.
+    // Persistent form (one workgroup per CU streams through its tiles) when its conditions hold
+    // (2-D tile order, at least 4 k-tiles, whole 16-byte output chunks, tiles under 2 GiB) and K is
+    // short enough for the tile switch to matter.  Measured: +3-12 % up to K = 4096, even at
+    // 8192, -2 % at K = 14336, where the fixed pairing of workgroups and tiles lets the
+    // workgroups of an XCD drift apart over the rounds and share less in L2 (+13 % HBM reads).
     bool persist = gnx == 4 && K / BK >= 4 && ncols % 8 == 0 && reinterpret_cast<uintptr_t>(Y) % 16 == 0 &&
                    ncols * (2 * BM) < (int64_t{1} << 31) && cus >= 8 && cus % 8 == 0;
-    if (const char *v = std::getenv("OPMX_MOE_GEMM_PERSIST")) persist = persist && std::atoi(v) != 0;   // tuning knob
+    if (const char *v = std::getenv("OPMX_MOE_GEMM_PERSIST")) {   // tuning knob: 0 = never, 1 = whenever possible
+        if (std::atoi(v) == 0) persist = false;
+    } else if (K / BK > 128) {
+        persist = false;
+    }
     if (persist) {
         const int smem_p = smem + 4 * 16 * (sw ? BN / 4 : BN / 2) * 2;       // + the four staging regions
         static bool attr_p[4] = {false, false, false, false};
