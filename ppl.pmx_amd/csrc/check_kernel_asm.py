@@ -11,8 +11,8 @@ checked on its output instead:
 2. no buffer load sits in a loop over lanes (a descriptor the compiler cannot prove uniform), and
    nothing spills to scratch memory inside the k loop: both would add memory operations the
    hand-written `s_waitcnt vmcnt(N)` counts know nothing about;
-3. the k loop (the innermost loop with the most MFMAs) holds exactly the MFMAs, LDS reads and
-   loads of one k-tile;
+3. the k loop (the loop with the most MFMAs, by the compiler's loop annotations) holds exactly
+   the MFMAs, LDS reads and loads of one k-tile;
 4. the persistent kernel issues the number of output stores per tile that its wait counts assume,
    and its tile loop has no scratch access and no wait that would drain the pipeline.
 
@@ -39,12 +39,46 @@ def functions(lines):
                 body.append(ln)
 
 
+def blocks(body):
+    """Splits a function body into basic blocks using the compiler's own annotations: returns
+    (instructions, per-instruction innermost loop header or None, parent header of each header,
+    headers of loops without inner loops)."""
+    text, where, parent, innermost = [], [], {}, set()
+    cur = None            # innermost loop header of the current block
+    pending_label = None
+    for raw in body:
+        line = raw.strip()
+        m = re.match(r"^(?:\.LBB\d+_(\d+):|; %bb\.(\d+):)\s*(;.*)?$", line)
+        if m:
+            pending_label = m.group(1) or m.group(2)
+            cur = None
+            line = m.group(3) or ""
+        if line.startswith(";"):
+            if pending_label is not None:
+                h = re.search(r"in Loop: Header=BB\d+_(\d+) Depth=\d+", line)
+                if h:
+                    cur = h.group(1)
+                if re.search(r"This (Inner )?Loop Header: Depth=\d+", line):
+                    cur = pending_label
+                    if "Inner" in line:
+                        innermost.add(pending_label)
+                pl = re.findall(r"Parent Loop BB\d+_(\d+) Depth=\d+", line)
+                if pl:
+                    parent.setdefault(pending_label, []).extend(pl)
+            continue
+        if not line:
+            continue
+        text.append(line)
+        where.append(cur)
+    # the innermost parent is the last "Parent Loop" line of a header
+    return text, where, {h: ps[-1] for h, ps in parent.items()}, innermost
+
+
 def check(path):
     findings, seen = [], 0
     for name, body in functions(open(path).read().split("\n")):
         seen += 1
-        code = [(i, l.strip()) for i, l in enumerate(body) if l.strip() and not l.strip().startswith(";")]
-        text = [l for _, l in code]
+        text, where, parent, innermost = blocks(body)
         mfma = [k for k, l in enumerate(text) if l.startswith("v_mfma")]
         nops = [k for k, l in enumerate(text) if l.startswith("s_nop 15")]
         if not mfma or not nops:
@@ -65,16 +99,14 @@ def check(path):
             if l.startswith("buffer_load") and " lds" in l and k and text[k - 1].startswith("s_and_saveexec"):
                 findings.append((name, "direct-to-LDS load inside a loop over lanes"))
                 break
-        # 2b/3. the k loop: the innermost loop holding the most MFMAs
-        labels = {l.split(":")[0]: k for k, l in enumerate(text) if re.match(r"^\.LBB\d+_\d+:", l)}
-        spans = []
-        for k, l in enumerate(text):
-            m = re.match(r"^s_cbranch_\w+ (\.LBB\d+_\d+)", l)
-            if m and labels.get(m.group(1), k + 1) <= k:          # a backward branch closes a loop
-                spans.append((labels[m.group(1)], k))
-        inner = [(a, z) for a, z in spans if not any((a2, z2) != (a, z) and a <= a2 and z2 <= z for a2, z2 in spans)]
-        kspan = max(inner, key=lambda t: sum(x.startswith("v_mfma") for x in text[t[0]:t[1] + 1]), default=(0, -1))
-        kloop = text[kspan[0]:kspan[1] + 1]
+        # 2b/3. the k loop: the innermost loop with the most MFMAs
+        per_loop = {}
+        for l, h in zip(text, where):
+            if h is not None:
+                per_loop.setdefault(h, []).append(l)
+        khead = max((h for h in per_loop if h in innermost),
+                    key=lambda h: sum(x.startswith("v_mfma") for x in per_loop[h]), default=None)
+        kloop = per_loop.get(khead, [])
         count = lambda p: sum(x.startswith(p) for x in kloop)
         if (count("v_mfma"), count("ds_read_b128"), count("buffer_load_dwordx4")) != (128, 32, 16):
             findings.append((name, "k loop holds {} MFMAs, {} LDS reads, {} loads (expected 128, 32, 16)".format(
@@ -85,18 +117,24 @@ def check(path):
         #    tile (16 or 32), the same number of priming stores before the tile loop, and no other
         #    store in the loop
         if "persist" in name:
-            outer = [(a, z) for a, z in spans if a <= kspan[0] and kspan[1] <= z and (a, z) != kspan]
-            if not outer:
+            thead = parent.get(khead)
+            if thead is None:
                 findings.append((name, "no loop over tiles found"))
             else:
-                a, z = min(outer, key=lambda t: t[1] - t[0])
+                def inside(h):
+                    while h is not None:
+                        if h == thead:
+                            return True
+                        h = parent.get(h)
+                    return False
+                tile = [l for l, h in zip(text, where) if inside(h)]
+                rest = [l for l, h in zip(text, where) if not inside(h)]
                 st = lambda part: sum(x.startswith("buffer_store_dwordx4") for x in part)
-                before, inside = st(text[:a]), st(text[a:z + 1])
-                if before not in (16, 32) or inside != before or st(text[z + 1:]) != 0:
-                    findings.append((name, "{} priming stores, {} stores in the tile loop".format(before, inside)))
+                if st(rest) not in (16, 32) or st(tile) != st(rest):
+                    findings.append((name, "{} priming stores, {} stores in the tile loop".format(st(rest), st(tile))))
                 # ... and that nothing in the tile loop drains the loads and stores kept in flight
                 # across tiles: no scratch traffic, no wait for all vector-memory operations
-                for l in text[a:z + 1]:
+                for l in tile:
                     if l.startswith("scratch_") or re.match(r"s_waitcnt .*vmcnt\(0\)", l):
                         findings.append((name, "in the tile loop: " + l))
     if seen == 0:

@@ -23,10 +23,10 @@ def test_checker_flags_a_copy_behind_an_mfma(tmp_path):
     import sys
     sys.path.insert(0, CSRC)
     import check_kernel_asm as C
-    good = ["_Z4x22gemm_tiled_dlds_kernelIfE:", ".LBB0_1:"] + \
+    good = ["_Z4x22gemm_tiled_dlds_kernelIfE:", ".LBB0_1:            ; =>This Inner Loop Header: Depth=1"] + \
         ["\tv_mfma_f32_16x16x32_f16 a[0:3], v[0:3], v[4:7], a[0:3]"] * 128 + \
         ["\tds_read_b128 v[0:3], v9"] * 32 + ["\tbuffer_load_dwordx4 v1, s[0:3], 0 offen lds"] * 16 + \
-        ["\ts_cbranch_scc1 .LBB0_1", "\ts_nop 15", "\tv_accvgpr_read_b32 v1, a0", ".Lfunc_end0:"]
+        ["\ts_cbranch_scc1 .LBB0_1", "; %bb.2:", "\ts_nop 15", "\tv_accvgpr_read_b32 v1, a0", ".Lfunc_end0:"]
     p = tmp_path / "good.s"
     p.write_text("\n".join(good))
     assert C.check(str(p)) == (1, [])
