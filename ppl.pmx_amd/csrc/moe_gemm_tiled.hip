@@ -207,12 +207,39 @@ __device__ __forceinline__ void locate_expert_major(int64_t lin, bool grouped, c
     }
 }
 
+// Row-partition order (gnx = 16), for column-tile counts that do not divide by 8 (11 column tiles
+// of the fine-grained gate/up GEMM): XCD x (ids = x mod 8) owns the row tiles
+// [x*mtiles/8, (x+1)*mtiles/8) with ALL their column tiles, and walks them four rows at a time:
+// for each group of four rows, for each column, the rows of the group -- its 32 resident
+// workgroups cover 4 rows x 8 columns.  Every expert's W is read by the one or two XCDs that own
+// its rows (in row-major order all eight read all of it).  XCDs own mtiles/8 row tiles rounded
+// down or up, so up to 8 * ntiles_n ids past the shorter ones name no tile (tile_m >= mtiles).
+__device__ __forceinline__ void map_row_partition(int64_t lin, int mtiles, int ntiles_n, int &tile_m, int &tile_n)
+{
+    const uint32_t xcd = static_cast<uint32_t>(lin) & 7, s = static_cast<uint32_t>(lin >> 3);
+    const uint32_t lo = xcd * static_cast<uint32_t>(mtiles) / 8, hi = (xcd + 1) * static_cast<uint32_t>(mtiles) / 8;
+    const uint32_t rows = hi - lo, per_group = 4u * static_cast<uint32_t>(ntiles_n);
+    tile_m = mtiles;
+    tile_n = 0;
+    if (s >= rows * static_cast<uint32_t>(ntiles_n)) return;
+    const uint32_t grp = s / per_group, t = s - grp * per_group;
+    const uint32_t h = rows - 4 * grp < 4 ? rows - 4 * grp : 4;
+    const uint32_t c = t / h;
+    tile_m = static_cast<int>(lo + 4 * grp + (t - c * h));
+    tile_n = static_cast<int>(c);
+}
+
 // Linear tile id -> tile, in whichever order gnx names.  mt.rows == 0: the id names no work.
 __device__ __forceinline__ void locate_any(int64_t lin, int gnx, int mtiles, int ntiles_n, bool grouped,
                                            const int64_t *s_off, int E, int64_t R, int BM, MTile &mt, int &tile_n)
 {
     if (gnx == 8) {
         locate_expert_major(lin, grouped, s_off, E, R, BM, ntiles_n, mt, tile_n);
+    } else if (gnx == 16) {
+        int tile_m;
+        map_row_partition(lin, mtiles, ntiles_n, tile_m, tile_n);
+        if (tile_m >= mtiles || tile_n >= ntiles_n) tile_m = -1;
+        row_tile(tile_m, grouped, s_off, E, R, BM, mt);
     } else {
         int tile_m;
         map_tile(static_cast<int>(lin), gnx, mtiles, ntiles_n, tile_m, tile_n);
@@ -225,16 +252,17 @@ __device__ __forceinline__ void locate_any(int64_t lin, int gnx, int mtiles, int
 inline int pick_gnx(int ntiles_n)
 {
     // XCD-grouped orders only when the n-tiles split evenly over the XCDs (else XCDs idle)
-    int gnx = ntiles_n % 8 == 0 ? 8 : 0;
+    int gnx = ntiles_n % 8 == 0 ? 8 : 16;
     if (const char *v = std::getenv("OPMX_MOE_GEMM_GNX")) gnx = std::atoi(v);   // tuning knob
-    if (gnx != 0 && gnx != 1 && gnx != 2 && gnx != 4 && gnx != 8) gnx = 0;
+    if (gnx != 0 && gnx != 1 && gnx != 2 && gnx != 4 && gnx != 8 && gnx != 16) gnx = 0;
     if (gnx == 4 && ntiles_n % 16 != 0) gnx = 0;
-    if (gnx != 0 && ntiles_n % 8 != 0) gnx = 0;
+    if (gnx != 0 && gnx != 16 && ntiles_n % 8 != 0) gnx = 0;
     return gnx;
 }
 inline int64_t linear_ids(int gnx, int ntiles_m, int ntiles_n)
 {
     if (gnx == 8) return static_cast<int64_t>(ntiles_n) * ntiles_m;     // exactly the tiles
+    if (gnx == 16) return 8 * ceil_div(ntiles_m, 8) * ntiles_n;          // every XCD as long as the longest
     if (gnx == 4) return ceil_div(ntiles_n, 16) * ceil_div(ntiles_m, 16) * 256;
     if (gnx > 0) return ceil_div(ntiles_n, 8 * gnx) * ceil_div(ntiles_m, 32 / gnx) * 256;
     return static_cast<int64_t>(ntiles_n) * ntiles_m;

@@ -106,6 +106,23 @@ def test_tile_order_with_partial_last_round(variant):
     run_case("row", [4096], 192, 4096, torch.float16, False, env)          # exactly one full round
 
 
+@pytest.mark.parametrize("variant", ["0", "1"])
+def test_expert_major_and_row_partition_tile_orders(variant):
+    """Tile orders of the 256-row kernels.  Expert-major (column tiles divisible by 8): experts
+    with 16-row-tile bands plus leftovers (4200 rows = 17 tiles, 5000 = 20), empty and one-row
+    experts, 8 and 24 column tiles.  Row partition (any other column-tile count): 3 and 11 column
+    tiles, more and fewer row tiles than XCDs.  Every tile must be computed exactly once: the
+    output starts out uninitialised."""
+    env = {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": variant}
+    big = [4200, 0, 300, 5000, 17, 256, 1, 2100]
+    run_case("column", big, 128, 2048, torch.float16, True, env)
+    run_case("row", big, 64, 6144, torch.bfloat16, False, env)
+    run_case("column", big, 128, 4096, torch.float16, False, env, swiglu=True)    # 16 column tiles of 128
+    run_case("column", big, 64, 768, torch.float16, True, env)                   # 3 column tiles
+    run_case("row", [300, 0, 129], 128, 2816, torch.bfloat16, False, env)         # 11 column tiles, 4 row tiles
+    run_case("column", [70] * 19, 64, 2816, torch.float16, False, env, swiglu=True)   # 19 row tiles, 11 column tiles of 128
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_persistent_kernel_streams_tiles(dtype):
     """The persistent form of the 256x256 kernel (16 column tiles, K >= 256): fewer tiles than
