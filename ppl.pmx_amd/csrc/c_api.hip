@@ -82,8 +82,13 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
         return launch_gemm_stream(X, off, W, B, E, R, K, N, dtype, epilogue, hint,
                                   env_int("OPMX_MOE_GEMM_STREAM_VARIANT", 0), Y, s);
     if (choice == 2) {
-        // 256x256 direct-to-LDS tiles from 128 mean rows per expert on, else 128x128 (measured).
-        const int dflt = R / E >= 128 ? 0 : 2;
+        // Direct-to-LDS kernel from 128 mean rows per expert on, else 128x128 register-staged
+        // (measured).  The direct-to-LDS kernel takes 256x256 tiles unless they would fill the CUs
+        // less than twice (the Mixtral down projection at T=2048: 1.3 rounds): then 128x256 tiles,
+        // 20 % slower per flop but with half the quantisation (-9 % there).
+        const int64_t out_cols = epilogue == OPMX_EPILOGUE_SWIGLU ? N / 2 : N;
+        const int64_t tiles256 = (R / 256 + (E + 1) / 2) * ((out_cols + 255) / 256);
+        const int dflt = R / E >= 128 ? (tiles256 < 512 ? 3 : 0) : 2;
         return launch_gemm_tiled(X, off, W, B, E, R, K, N, dtype, epilogue,
                                  env_int("OPMX_MOE_GEMM_TILED_VARIANT", dflt), Y, ws, ws_bytes, s);
     }

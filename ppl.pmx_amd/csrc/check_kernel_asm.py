@@ -108,9 +108,11 @@ def check(path):
                     key=lambda h: sum(x.startswith("v_mfma") for x in per_loop[h]), default=None)
         kloop = per_loop.get(khead, [])
         count = lambda p: sum(x.startswith(p) for x in kloop)
-        if (count("v_mfma"), count("ds_read_b128"), count("buffer_load_dwordx4")) != (128, 32, 16):
-            findings.append((name, "k loop holds {} MFMAs, {} LDS reads, {} loads (expected 128, 32, 16)".format(
-                count("v_mfma"), count("ds_read_b128"), count("buffer_load_dwordx4"))))
+        # 256 x 256 tiles (template arguments <T, 256, 256, ...>) or 128 x 256
+        expected = (64, 24, 12) if "Li128ELi256E" in name else (128, 32, 16)
+        if (count("v_mfma"), count("ds_read_b128"), count("buffer_load_dwordx4")) != expected:
+            findings.append((name, "k loop holds {} MFMAs, {} LDS reads, {} loads (expected {}, {}, {})".format(
+                count("v_mfma"), count("ds_read_b128"), count("buffer_load_dwordx4"), *expected)))
         if any(x.startswith("scratch_") for x in kloop):
             findings.append((name, "scratch access inside the k loop"))
         # 4. persistent kernel: the wait counts assume a fixed number of output stores per wave and

@@ -628,12 +628,28 @@ __device__ __forceinline__ void barrier_no_fence()
     asm volatile("" ::: "memory");
 }
 
+// Where the LDS fragment reads and the global -> LDS loads of a k-tile step sit among its four
+// groups of MFMAs (OPMX_ITERX below).  `wide`: the wave tile has 8 column sub-tiles (128 x 128,
+// 32 MFMAs per group, 16 loads per step) or 4 (128 x 64, 16 MFMAs per group, 12 loads per step).
+__device__ __forceinline__ constexpr bool g0_reads(bool wide, int m) { return wide ? m % 2 == 0 : m < 12; }   // group 0: a read behind MFMA m?
+__device__ __forceinline__ constexpr int g0_slot(bool wide, int m) { return wide ? m / 2 : m; }               // ... which of the 8 + TNS reads
+__device__ __forceinline__ constexpr int g1_barrier(bool wide) { return wide ? 10 : 5; }                       // group 1: "buffer free" barrier
+__device__ __forceinline__ constexpr int g1_load(bool wide, int m)                                             // group 1: load behind MFMA m, or -1
+{
+    return wide ? ((m >= 11 && (m - 11) % 3 == 0) ? (m - 11) / 3 : -1) : ((m >= 6 && m % 2 == 0) ? (m - 6) / 2 : -1);
+}
+__device__ __forceinline__ constexpr int g2_load(bool wide, int m)                                             // group 2: the remaining loads
+{
+    return wide ? ((m % 3 == 0 && m / 3 < 9) ? 7 + m / 3 : -1) : ((m % 2 == 0 && m / 2 < 7) ? 5 + m / 2 : -1);
+}
+
 // Waits until at most N vector-memory operations of this wave are outstanding (they complete
 // in issue order, loads and stores alike).
 template <int N> __device__ __forceinline__ void wait_vm()
 {
-    static_assert(N == 0 || N == 16 || N == 32 || N == 48, "add the immediate here");
+    static_assert(N == 0 || N == 12 || N == 16 || N == 32 || N == 48, "add the immediate here");
     if (N == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (N == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
     if (N == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
     if (N == 32) asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
     if (N == 48) asm volatile("s_waitcnt vmcnt(48)" ::: "memory");
@@ -762,13 +778,15 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
                                                                int ntiles_n, int gnx, int sk_wgs, int sk_cost,
                                                                float *__restrict__ sk_part, int *__restrict__ sk_count)
 {
-    constexpr int WM = 2, WN = 2, NW = 4;
+    constexpr int NW = 4, WM = BM / 128, WN = NW / WM;                 // 256 x 256: 2 x 2 waves, 128 x 256: 1 x 4
     constexpr int WTM = BM / WM, WTN = BN / WN, TMS = WTM / 16, TNS = WTN / 16, HM = TMS / 2;
     constexpr int BNO = SWIGLU ? BN / 2 : BN;
     constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW, NL = LA + LB;   // 1 KiB wave loads per k-tile
     constexpr int STAGE = (BM + BN) * ROWB;
     constexpr int NM = HM * TNS;
-    static_assert(HM == 4 && TNS == 8 && NL == 16, "the schedule below is written for 128x128 wave tiles");
+    constexpr bool WIDE = TNS == 8;
+    static_assert(HM == 4 && ((TNS == 8 && NL == 16) || (TNS == 4 && NL == 12)),
+                  "the schedule below is written for 128x128 and 128x64 wave tiles");
     using frag = typename Mfma<T>::frag;
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -864,22 +882,22 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
     do {                                                                                           \
         _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
             OPMX_MF0(FIRST, 0, m);                                                                 \
-            if (m % 2 == 0) {                                                                      \
-                const int r = m / 2;                                                               \
+            if (g0_reads(WIDE, m)) {                                                               \
+                const int r = g0_slot(WIDE, m);                                                    \
                 if (r < 4) OPMX_XFRAG(B, 0, 1, r < 4 ? r : 0);                                     \
                 else if (r < 8) OPMX_XFRAG(B, 1, 0, (r >= 4 && r < 8) ? r - 4 : 0);                \
-                else OPMX_WFRAG(B, 1, r >= 8 ? r - 8 : 0);                                         \
+                else OPMX_WFRAG(B, 1, (r >= 8 && r < 8 + TNS) ? r - 8 : 0);                        \
             }                                                                                      \
         }                                                                                          \
         _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
             OPMX_MF0(FIRST, 1, m);                                                                 \
             if (m < 4) OPMX_XFRAG(B, 1, 1, m < 4 ? m : 0);                                         \
-            if (m == 10) barrier_no_fence();                                                       \
-            if ((LD2) && m >= 11 && (m - 11) % 3 == 0) OPMX_ISSUE1(LDK, B, (m - 11) / 3);          \
+            if (m == g1_barrier(WIDE)) barrier_no_fence();                                         \
+            if ((LD2) && g1_load(WIDE, m) >= 0) OPMX_ISSUE1(LDK, B, g1_load(WIDE, m) >= 0 ? g1_load(WIDE, m) : 0); \
         }                                                                                          \
         _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
             OPMX_MF(1, 0, m);                                                                      \
-            if ((LD2) && m % 3 == 0 && m / 3 < 9) OPMX_ISSUE1(LDK, B, 7 + m / 3);                  \
+            if ((LD2) && g2_load(WIDE, m) >= 0) OPMX_ISSUE1(LDK, B, g2_load(WIDE, m) >= 0 ? g2_load(WIDE, m) : 0); \
         }                                                                                          \
         wait_vm<(LD2) ? (VM) : 0>();                                                               \
         __builtin_amdgcn_s_barrier();                                                              \
@@ -887,10 +905,10 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
         _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
             OPMX_MF(1, 1, m);                                                                      \
             if ((NEXT) && m < 4) OPMX_XFRAG((B) ^ 1, 0, 0, m < 4 ? m : 0);                         \
-            else if ((NEXT) && m < 12) OPMX_WFRAG((B) ^ 1, 0, (m >= 4 && m < 12) ? m - 4 : 0);     \
+            else if ((NEXT) && m < 4 + TNS) OPMX_WFRAG((B) ^ 1, 0, (m >= 4 && m < 4 + TNS) ? m - 4 : 0); \
         }                                                                                          \
     } while (0)
-#define OPMX_ITER(KT, B, LD2, NEXT) OPMX_ITERX((KT) + 2, B, LD2, NEXT, false, 16)
+#define OPMX_ITER(KT, B, LD2, NEXT) OPMX_ITERX((KT) + 2, B, LD2, NEXT, false, NL)
 
     // prologue: first k-tile -> buffer 0, second -> buffer 1, wait for the first
 #pragma unroll
@@ -898,7 +916,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
     if (kt1 - kt0 > 1) {
 #pragma unroll
         for (int q = 0; q < NL; ++q) OPMX_ISSUE1(kt0 + 1, 1, q);
-        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+        wait_vm<NL>();
     } else {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
@@ -1120,6 +1138,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
     constexpr int NS = WTM * (SWIGLU ? WTN / 2 : WTN) * 2 / 1024;      // output stores per wave and tile
     static_assert(HM == 4 && TNS == 8 && NL == 16, "the schedule is written for 128x128 wave tiles");
     constexpr int NOB = SWIGLU ? TNS / 2 : TNS;                       // output sub-tile columns per wave
+    constexpr bool WIDE = true;
     static_assert(NS == 16 || NS == 32, "wait counts below");
     using frag = typename Mfma<T>::frag;
 
@@ -1318,7 +1337,7 @@ template <typename T, int BM, int BN>
 int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
                       int64_t K, int64_t N, int epilogue, void *Y, void *ws, size_t ws_bytes, hipStream_t s)
 {
-    static_assert(BM * BN == kSkTile, "tail slot size");
+    static_assert(BM * BN <= kSkTile, "tail slot size");
     constexpr int smem = 2 * (BM + BN) * ROWB;
     const bool sw = epilogue == OPMX_EPILOGUE_SWIGLU;
     const int64_t ncols = sw ? N / 2 : N;
@@ -1371,7 +1390,7 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
     } else if (K / BK > 128) {
         persist = false;
     }
-    if (persist) {
+    if constexpr (BM == 256) if (persist) {
         const int smem_p = smem + 4 * 16 * (sw ? BN / 4 : BN / 2) * 2;       // + the four staging regions
         static bool attr_p[4] = {false, false, false, false};
         const bool hb = B != nullptr;
@@ -1428,6 +1447,7 @@ int tiled_impl(const void *X, const int64_t *off, const void *W, const void *B, 
     switch (variant) {
         case 1: return tiled_launch<T, 256, 256, 2, 4>(X, off, W, B, E, R, K, N, epilogue, Y, s);
         case 2: return tiled_launch<T, 128, 128, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        case 3: return tiled_dlds_launch<T, 128, 256>(X, off, W, B, E, R, K, N, epilogue, Y, ws, ws_bytes, s);
         default: return tiled_dlds_launch<T, 256, 256>(X, off, W, B, E, R, K, N, epilogue, Y, ws, ws_bytes, s);
     }
 }

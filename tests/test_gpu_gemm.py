@@ -83,7 +83,7 @@ def test_tiny_config_fp32_shapes():
     run_case("column", sizes, 1024, 5632, torch.float32, True, swiglu=True)
 
 
-@pytest.mark.parametrize("variant", ["0", "1", "2"])
+@pytest.mark.parametrize("variant", ["0", "1", "2", "3"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_tiled_kernel_variants(variant, dtype):
     env = {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": variant}
@@ -95,7 +95,7 @@ def test_tiled_kernel_variants(variant, dtype):
     run_case("column", sizes, 64, 1000, dtype, False, env, swiglu=True)   # D=500: ragged epilogue tile
 
 
-@pytest.mark.parametrize("variant", ["0", "1", "2"])
+@pytest.mark.parametrize("variant", ["0", "1", "2", "3"])
 def test_tile_order_with_partial_last_round(variant):
     """16 column tiles and 24 row tiles: one full 16 x 16 round in the XCD-grouped order plus
     eight row tiles dealt out by the remainder rule; SwiGLU case: 16 column tiles of 128."""
@@ -106,7 +106,7 @@ def test_tile_order_with_partial_last_round(variant):
     run_case("row", [4096], 192, 4096, torch.float16, False, env)          # exactly one full round
 
 
-@pytest.mark.parametrize("variant", ["0", "1"])
+@pytest.mark.parametrize("variant", ["0", "1", "3"])
 def test_expert_major_and_row_partition_tile_orders(variant):
     """Tile orders of the 256-row kernels.  Expert-major (column tiles divisible by 8): experts
     with 16-row-tile bands plus leftovers (4200 rows = 17 tiles, 5000 = 20), empty and one-row
@@ -155,6 +155,8 @@ def test_tail_tiles_split_over_k(dtype):
     assert torch.equal(a, b)
     c = run_case("row", sizes, 2048, 4096, dtype, True, dict(env, OPMX_MOE_GEMM_STREAMK="0"))
     assert (a.float() - c.float()).abs().max() <= 2e-2 * max(1.0, float(c.float().abs().max()))
+    # the 128 x 256 tile form of the kernel (half-size partial tiles)
+    run_case("row", sizes, 2048, 4096, dtype, True, dict(env, OPMX_MOE_GEMM_TILED_VARIANT="3"))
     # a K long enough for the default policy to split (144 k-tiles, 8 ranges)
     if dtype == torch.float16:
         run_case("row", [200, 60], 9216, 4096, dtype, False, {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": "0"})
