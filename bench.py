@@ -76,6 +76,8 @@ def main():
                     help="skip the probe of the HBM-read / MFMA rates this device sustains")
     ap.add_argument("--no-vendor-gemm", action="store_true",
                     help="MFMA-bound workloads: skip timing the vendor dense GEMM of the same flop count")
+    ap.add_argument("--no-companion", action="store_true",
+                    help="with the default workload, do not also measure the MFMA-bound prefill workload")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
                     help="also run N plain device-to-device copies of the gate/up weight tensor (known size): "
                          "the reference reading for FETCH_SIZE / WRITE_SIZE counter runs")
@@ -99,6 +101,24 @@ def main():
                                                  check=True).stdout.strip().splitlines()[-1])
         except Exception as exc:   # the probe is optional
             print("device ceiling probe failed: {}".format(exc), file=sys.stderr)
+    # The default run (decode, HBM-bound) also reports the MFMA-bound companion workload of the
+    # same layer, prefill T=8192 with skewed routing, as six operators and with the SwiGLU
+    # epilogue: child processes of this program, run while this one leaves the GPU idle.
+    companion = None
+    if args.workload == "decode-T32" and not args.no_companion:
+        import subprocess
+        companion = {}
+        for name, extra in (("prefill-T8192", []), ("prefill-T8192, fused SwiGLU epilogue", ["--fuse-swiglu"])):
+            cmd = [sys.executable, os.path.abspath(__file__), "--workload", "prefill-T8192", "--steps", "50", "--warmup", "5",
+                   "--no-cpu-baseline", "--no-device-ceilings", "--no-vendor-gemm", "--no-companion"] + extra
+            try:
+                line = subprocess.run(cmd, capture_output=True, text=True, timeout=300, check=True).stdout.strip().splitlines()[-1]
+                r = json.loads(line)
+                companion[name] = {key: r[key] for key in ("value", "unit", "ms_per_step", "steps", "config", "roofline",
+                                                           "layer", "per_op_us")}
+            except Exception as exc:
+                print("companion workload failed: {}".format(exc), file=sys.stderr)
+
     import torch_function as OPMX
     from model_zoo.mixtral.modeling.dynamic_batching.Model import MoeFeedForward
 
@@ -259,7 +279,7 @@ def main():
             "path": "drop-in operator sequence" + (" + fused SwiGLU epilogue" if args.fuse_swiglu else ""),
             "active_experts": active, "max_expert_share": round(float(counts.max()) / R, 3)},
         "roofline": roof, "layer": lay, "per_op_us": {n: round(v, 1) for n, v in per_op.items()},
-        "device_ceilings": ceilings, "vendor_dense_gemm_same_flops_TFLOPs": vendor_tflops, "device": torch.cuda.get_device_name(0), "cu_count": torch.cuda.get_device_properties(0).multi_processor_count,
+        "device_ceilings": ceilings, "companion": companion, "vendor_dense_gemm_same_flops_TFLOPs": vendor_tflops, "device": torch.cuda.get_device_name(0), "cu_count": torch.cuda.get_device_properties(0).multi_processor_count,
     }
 
     # ---- CPU baseline: the oracle (PyTorch CPU restatement of the reference operator
