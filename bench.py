@@ -44,7 +44,7 @@ MFMA_PEAK_TFLOPS = 2500.0      # dense fp16/bf16 MFMA, vendor figure
 # profiles/gemm_tiled_prefill_T8192_mixtral8x7b.txt.  None where no counter run was made.
 MEASURED_TRAFFIC = {
     ("decode-T32", False): 1883442790 + 3759718,
-    ("prefill-T8192", False): 2 * 4051123 * 1024 + 917504 * 1024,
+    ("prefill-T8192", False): 2 * 4160709 * 1024 + 917504 * 1024,
 }
 
 SHAPES = {
