@@ -63,16 +63,15 @@ __device__ __forceinline__ int count_mtiles(bool grouped, const int64_t *s_off, 
     return __builtin_amdgcn_readfirstlane(static_cast<int>(total));
 }
 
-// Linear tile id -> (row tile, column tile); mtiles is the actual number of row tiles.
-// Workgroups are handed to the 8 XCDs round-robin by linear id and each XCD has its own L2, so
-// 256 consecutive ids ("a round", 32 per XCD) form a block of tiles in which every XCD owns a
-// compact sub-block: its 32 resident workgroups then share X- and W-tiles in that XCD's L2.
-//   gnx = 1, 2: XCDs side by side along n, each (32/gnx) x gnx tiles;
-//   gnx = 4   : rounds of 16 x 16 tiles, XCDs as 2 (m) x 4 (n), each 8 x 4 tiles (a third less
-//               L2 fill traffic than 16 x 2).  The last mtiles % 16 row tiles would leave XCDs
-//               idle in that layout; they are dealt out differently: XCD j takes the column
-//               tiles [j*ntiles_n/8, (j+1)*ntiles_n/8), walking m fastest.  ntiles_n % 16 == 0.
-//   gnx = 0   : plain row-major order, n fastest.
+// Linear tile id -> (row tile, column tile) over the row tiles of all experts strung together;
+// mtiles is the actual number of row tiles.  Workgroups are handed to the 8 XCDs round-robin by
+// linear id and each XCD has its own L2, so the order of the ids decides which tiles share an L2.
+//   gnx = 4: rounds of 16 x 16 tiles, XCDs as 2 (m) x 4 (n), each a compact 8 x 4 sub-block (a
+//            third less L2 fill traffic than 16 x 2).  The last mtiles % 16 row tiles would leave
+//            XCDs idle in that layout; XCD j takes their column tiles [j*ntiles_n/8, (j+1)*ntiles_n/8),
+//            walking m fastest.  ntiles_n % 16 == 0.  Kept as the comparison point of the
+//            expert-major order below, which replaced it.
+//   gnx = 0: plain row-major order, n fastest.
 // Ids that name no tile come back with tile_m >= mtiles.
 __device__ __forceinline__ void map_tile(int lin, int gnx, int mtiles, int ntiles_n, int &tile_m, int &tile_n)
 {
@@ -93,11 +92,6 @@ __device__ __forceinline__ void map_tile(int lin, int gnx, int mtiles, int ntile
                 tile_n = 0;
             }
         }
-    } else if (gnx > 0) {
-        const int gm = 32 / gnx;
-        const int rounds_n = (ntiles_n + 8 * gnx - 1) / (8 * gnx);
-        tile_m = (round / rounds_n) * gm + sl % gm;
-        tile_n = (round % rounds_n) * (8 * gnx) + xcd * gnx + sl / gm;
     } else {
         tile_m = lin / ntiles_n;
         tile_n = lin % ntiles_n;
@@ -254,9 +248,9 @@ inline int pick_gnx(int ntiles_n)
     // XCD-grouped orders only when the n-tiles split evenly over the XCDs (else XCDs idle)
     int gnx = ntiles_n % 8 == 0 ? 8 : 16;
     if (const char *v = std::getenv("OPMX_MOE_GEMM_GNX")) gnx = std::atoi(v);   // tuning knob
-    if (gnx != 0 && gnx != 1 && gnx != 2 && gnx != 4 && gnx != 8 && gnx != 16) gnx = 0;
+    if (gnx != 0 && gnx != 4 && gnx != 8 && gnx != 16) gnx = 0;
     if (gnx == 4 && ntiles_n % 16 != 0) gnx = 0;
-    if (gnx != 0 && gnx != 16 && ntiles_n % 8 != 0) gnx = 0;
+    if (gnx == 8 && ntiles_n % 8 != 0) gnx = 0;
     return gnx;
 }
 inline int64_t linear_ids(int gnx, int ntiles_m, int ntiles_n)
@@ -264,7 +258,6 @@ inline int64_t linear_ids(int gnx, int ntiles_m, int ntiles_n)
     if (gnx == 8) return static_cast<int64_t>(ntiles_n) * ntiles_m;     // exactly the tiles
     if (gnx == 16) return 8 * ceil_div(ntiles_m, 8) * ntiles_n;          // every XCD as long as the longest
     if (gnx == 4) return ceil_div(ntiles_n, 16) * ceil_div(ntiles_m, 16) * 256;
-    if (gnx > 0) return ceil_div(ntiles_n, 8 * gnx) * ceil_div(ntiles_m, 32 / gnx) * 256;
     return static_cast<int64_t>(ntiles_n) * ntiles_m;
 }
 
