@@ -35,6 +35,15 @@ template <typename T> __device__ __forceinline__ void store16(T *p, const Vec16<
 {
     *reinterpret_cast<uint4 *>(p) = *reinterpret_cast<const uint4 *>(&r);
 }
+// The same for data that is read once: a load the caches need not keep.
+template <typename T> __device__ __forceinline__ Vec16<T> load16_once(const T *p)
+{
+    typedef uint32_t quad __attribute__((ext_vector_type(4)));
+    Vec16<T> r;
+    const quad q = __builtin_nontemporal_load(reinterpret_cast<const quad *>(p));
+    __builtin_memcpy(&r, &q, 16);
+    return r;
+}
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
 
