@@ -84,7 +84,12 @@ int linear_impl(const void *X_, const void *W_, const void *B_, int64_t Ttok, in
     const T *X = static_cast<const T *>(X_), *W = static_cast<const T *>(W_), *B = static_cast<const T *>(B_);
     T *Y = static_cast<T *>(Y_);
     const bool vec = K % Vec16<T>::n == 0 && aligned16(X) && aligned16(W);
-    if (Ttok >= 1024) {
+    if (Ttok >= 4096) {
+        // 8 tokens per block: W (read from cache by every block) is amortised over more rows of X
+        const dim3 grid(static_cast<unsigned>(ceil_div(Ttok, 8)), static_cast<unsigned>(ceil_div(N, kNT)));
+        if (vec) linear_kernel<T, 8, true><<<grid, 256, 0, s>>>(X, W, B, Ttok, K, N, Y);
+        else linear_kernel<T, 8, false><<<grid, 256, 0, s>>>(X, W, B, Ttok, K, N, Y);
+    } else if (Ttok >= 1024) {
         const dim3 grid(static_cast<unsigned>(ceil_div(Ttok, 4)), static_cast<unsigned>(ceil_div(N, kNT)));
         if (vec) linear_kernel<T, 4, true><<<grid, 256, 0, s>>>(X, W, B, Ttok, K, N, Y);
         else linear_kernel<T, 4, false><<<grid, 256, 0, s>>>(X, W, B, Ttok, K, N, Y);
