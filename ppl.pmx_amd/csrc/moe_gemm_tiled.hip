@@ -1105,7 +1105,7 @@ __device__ __forceinline__ void tile_epilogue_staged_impl(
 }
 
 // Persistent form of gemm_tiled_dlds_kernel: one workgroup per CU walks the tile ids
-// blockIdx.x, blockIdx.x + gridDim.x, ... (2-D tile order only, K >= 4 k-tiles) and treats them
+// blockIdx.x, blockIdx.x + gridDim.x, ... (XCD-aware tile orders only, K >= 4 k-tiles) and treats them
 // as one continuous stream of k-tiles.  The last two k-tile steps of a tile already load the
 // first two k-tiles of the next one, so there is no pipeline refill between tiles, and the
 // output stores of a tile drain behind the MFMAs of the next: they are issued after those loads,
@@ -1145,7 +1145,11 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
     const int nk = static_cast<int>(K / BK);
     const int64_t ttot = static_cast<int64_t>(mtiles) * ntiles_n;
     const int g = sk_split(ttot, sk_wgs, nk, gnx, sk_cost);
-    const int64_t nmain = g > 1 ? ttot - ttot % sk_wgs : ttot;        // ids [nmain, ttot) are the tail launch's
+    // ids [nmain, ttot) are the tail launch's.  The row-partition order has ids that name no tile
+    // behind the last tile of each XCD: its id space is longer than the tile count, and a
+    // workgroup's stream ends at the first such id (all later ones of its XCD are empty too).
+    const int64_t ids = gnx == 16 ? int64_t{8} * ((mtiles + 7) / 8) * ntiles_n : ttot;
+    const int64_t nmain = g > 1 ? ttot - ttot % sk_wgs : ids;
     int64_t id = blockIdx.x;
     if (id >= nmain) return;
 
@@ -1376,7 +1380,7 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
     // short enough for the tile switch to matter.  Measured: +3-12 % up to K = 4096, even at
     // 8192, -2 % at K = 14336, where the fixed pairing of workgroups and tiles lets the
     // workgroups of an XCD drift apart over the rounds and share less in L2 (+13 % HBM reads).
-    bool persist = (gnx == 4 || gnx == 8) && K / BK >= 4 && ncols % 8 == 0 && reinterpret_cast<uintptr_t>(Y) % 16 == 0 &&
+    bool persist = (gnx == 4 || gnx == 8 || gnx == 16) && K / BK >= 4 && ncols % 8 == 0 && reinterpret_cast<uintptr_t>(Y) % 16 == 0 &&
                    ncols * (2 * BM) < (int64_t{1} << 31) && cus >= 8 && cus % 8 == 0;
     if (const char *v = std::getenv("OPMX_MOE_GEMM_PERSIST")) {   // tuning knob: 0 = never, 1 = whenever possible
         if (std::atoi(v) == 0) persist = false;

@@ -136,6 +136,10 @@ def test_persistent_kernel_streams_tiles(dtype):
         a = run_case("column", sizes, K, 4096, dtype, bias, env, swiglu=swiglu)
         b = run_case("column", sizes, K, 4096, dtype, bias, dict(env, OPMX_MOE_GEMM_PERSIST="0"), swiglu=swiglu)
         assert torch.equal(a, b)
+    # row-partition order (11 column tiles), several tiles per workgroup, uneven XCD shares (27 row tiles)
+    a = run_case("column", sizes, 256, 2816, dtype, True, env)
+    b = run_case("column", sizes, 256, 2816, dtype, True, dict(env, OPMX_MOE_GEMM_PERSIST="0"))
+    assert torch.equal(a, b)
     # with the tail of the last round split over k by the second launch
     run_case("row", sizes, 1024, 4096, dtype, True, dict(env, OPMX_MOE_GEMM_STREAMK="2"))
 
