@@ -76,8 +76,6 @@ def main():
                     help="skip the probe of the HBM-read / MFMA rates this device sustains")
     ap.add_argument("--no-vendor-gemm", action="store_true",
                     help="MFMA-bound workloads: skip timing the vendor dense GEMM of the same flop count")
-    ap.add_argument("--pretiled-weights", action="store_true",
-                    help="repack the expert weights once before timing (16x64 tiles, opmx_moe_retile_weights)")
     ap.add_argument("--no-companion", action="store_true",
                     help="with the default workload, do not also measure the MFMA-bound prefill workload")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
@@ -105,19 +103,14 @@ def main():
             print("device ceiling probe failed: {}".format(exc), file=sys.stderr)
     # The default run (decode, HBM-bound) also reports the MFMA-bound companion workload of the
     # same layer, prefill T=8192 with skewed routing, as six operators and with the SwiGLU
-    # epilogue, and the decode workload itself with the expert weights repacked at load time:
-    # child processes of this program, run while this one leaves the GPU idle.
+    # epilogue: child processes of this program, run while this one leaves the GPU idle.
     companion = None
     if args.workload == "decode-T32" and not args.no_companion:
         import subprocess
         companion = {}
-        for name, extra in (("prefill-T8192", ["--workload", "prefill-T8192", "--steps", "50"]),
-                            ("prefill-T8192, fused SwiGLU epilogue",
-                             ["--workload", "prefill-T8192", "--steps", "50", "--fuse-swiglu"]),
-                            ("decode-T32, expert weights repacked at load time",
-                             ["--workload", "decode-T32", "--steps", "200", "--pretiled-weights"])):
-            cmd = [sys.executable, os.path.abspath(__file__), "--warmup", "5", "--no-cpu-baseline", "--no-device-ceilings",
-                   "--no-vendor-gemm", "--no-companion"] + extra
+        for name, extra in (("prefill-T8192", []), ("prefill-T8192, fused SwiGLU epilogue", ["--fuse-swiglu"])):
+            cmd = [sys.executable, os.path.abspath(__file__), "--workload", "prefill-T8192", "--steps", "50", "--warmup", "5",
+                   "--no-cpu-baseline", "--no-device-ceilings", "--no-vendor-gemm", "--no-companion"] + extra
             try:
                 line = subprocess.run(cmd, capture_output=True, text=True, timeout=300, check=True).stdout.strip().splitlines()[-1]
                 r = json.loads(line)
@@ -149,13 +142,7 @@ def main():
         p = torch.arange(1, E + 1, dtype=torch.float64) ** -1.2
         bias = (cfg["skew"] * torch.log(p / p.sum())).to(dtype).to(dev)
         layer.gate.bias = torch.nn.Parameter(bias, requires_grad=False)
-    if args.pretiled_weights:
-        layer.retile_()
     Wg, wu, w2, gb = layer.gate.weight, layer.wu.weight, layer.w2.weight, layer.gate.bias
-    # the operators on the expert weights, for the layout the weights are in
-    lay_w = layer.wu.weight_layout
-    col = OPMX.moe_column_parallel_linear_tiled if args.pretiled_weights else OPMX.moe_column_parallel_linear
-    row = OPMX.moe_row_parallel_linear_tiled if args.pretiled_weights else OPMX.moe_row_parallel_linear
 
     # ---- one instrumented pass: routing statistics + per-operator durations
     def ops(record=None):
@@ -171,11 +158,11 @@ def main():
         sc = timed("router_linear", lambda: OPMX.linear(x, Wg, gb, H, E))
         xe, w, inv, off = timed("moe_select", lambda: OPMX.moe_select(x, sc, E, k))
         if args.fuse_swiglu:
-            act = timed("gate_up_gemm", lambda: OPMX.moe_column_parallel_linear_swiglu(xe, off, wu, None, E, H, 2 * I, lay_w))
+            act = timed("gate_up_gemm", lambda: OPMX.moe_column_parallel_linear_swiglu(xe, off, wu, None, E, H, 2 * I))
         else:
-            h = timed("gate_up_gemm", lambda: col(xe, off, wu, None, None, E, H, 2 * I, False))
+            h = timed("gate_up_gemm", lambda: OPMX.moe_column_parallel_linear(xe, off, wu, None, None, E, H, 2 * I, False))
             act = timed("swiglu", lambda: OPMX.swiglu(h))
-        y = timed("down_gemm", lambda: row(act, off, w2, None, None, E, I, H, True))
+        y = timed("down_gemm", lambda: OPMX.moe_row_parallel_linear(act, off, w2, None, None, E, I, H, True))
         out = timed("moe_reduce", lambda: OPMX.moe_reduce(y, w, inv, k))
         return out, off
 
@@ -191,9 +178,9 @@ def main():
 
         # ---- timed region: exactly --steps steps; HIP events bracket the dominant kernel
         ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-        gemm1 = (lambda xe, off: OPMX.moe_column_parallel_linear_swiglu(xe, off, wu, None, E, H, 2 * I, lay_w)) \
+        gemm1 = (lambda xe, off: OPMX.moe_column_parallel_linear_swiglu(xe, off, wu, None, E, H, 2 * I)) \
             if args.fuse_swiglu else \
-            (lambda xe, off: col(xe, off, wu, None, None, E, H, 2 * I, False))
+            (lambda xe, off: OPMX.moe_column_parallel_linear(xe, off, wu, None, None, E, H, 2 * I, False))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for i in range(args.steps):
@@ -203,7 +190,7 @@ def main():
             h = gemm1(xe, off)
             ev[i][1].record()
             act = h if args.fuse_swiglu else OPMX.swiglu(h)
-            y = row(act, off, w2, None, None, E, I, H, True)
+            y = OPMX.moe_row_parallel_linear(act, off, w2, None, None, E, I, H, True)
             out = OPMX.moe_reduce(y, w, inv, k)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
@@ -289,8 +276,7 @@ def main():
         "dtype": {"float16": "f16", "bfloat16": "bf16"}[cfg["dtype"]], "data": "synthetic",
         "config": {"workload": "{} MoE layer {}, T={} tokens, hidden={}, experts={}, top-{}, ffn={}, TP=1".format(
             cfg["name"], "decode" if hbm_bound else "prefill", T, H, E, k, I),
-            "path": "drop-in operator sequence" + (" + fused SwiGLU epilogue" if args.fuse_swiglu else "") +
-                    (", expert weights repacked into 16x64 tiles at load time" if args.pretiled_weights else ""),
+            "path": "drop-in operator sequence" + (" + fused SwiGLU epilogue" if args.fuse_swiglu else ""),
             "active_experts": active, "max_expert_share": round(float(counts.max()) / R, 3)},
         "roofline": roof, "layer": lay, "per_op_us": {n: round(v, 1) for n, v in per_op.items()},
         "device_ceilings": ceilings, "companion": companion, "vendor_dense_gemm_same_flops_TFLOPs": vendor_tflops, "device": torch.cuda.get_device_name(0), "cu_count": torch.cuda.get_device_properties(0).multi_processor_count,
@@ -301,8 +287,6 @@ def main():
     if not args.no_cpu_baseline:
         from oracle import moe_oracle as O
         Tc = T if T <= 512 else 512            # bounded sample of the same workload
-        if args.pretiled_weights:              # the oracle reads the reference layout
-            wu, w2 = (OPMX.moe_retile_weights(t, OPMX.WEIGHTS_ROW_MAJOR) for t in (wu, w2))
         xc, Wgc, wuc, w2c = x[:Tc].cpu(), Wg.cpu(), wu.cpu(), w2.cpu()
         gbc = None if gb is None else gb.cpu()
         def timed_runs(budget, **kw):

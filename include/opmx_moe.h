@@ -56,18 +56,6 @@ typedef enum opmx_epilogue {
     OPMX_EPILOGUE_SWIGLU = 1
 } opmx_epilogue;
 
-/* Memory layout of the expert weights W [E,N,K] of the grouped GEMM. */
-typedef enum opmx_weight_layout {
-    /* the reference's: W[e] is [N,K] row-major (model_zoo/ModelParallel.py:149-151,
-     * checkpoints of model_zoo/mixtral/huggingface/ConvertWeightToOpmx.py:98-128) */
-    OPMX_WEIGHTS_ROW_MAJOR = 0,
-    /* W[e] cut into tiles of 16 rows x 64 k, stored tile after tile, k fastest: element (n,k)
-     * at e*N*K + ((n/16)*(K/64) + k/64)*1024 + (n%16)*64 + k%64.  The 16 weight rows a wave
-     * streams are then one contiguous run: +7-9 % decode bandwidth.  f16/bf16, N % 16 == 0
-     * (and (N/2) % 16 == 0 with the SwiGLU epilogue), K % 64 == 0. */
-    OPMX_WEIGHTS_TILED_16X64 = 1
-} opmx_weight_layout;
-
 /* Limits of the routing kernels. */
 #define OPMX_MOE_MAX_EXPERTS 256
 #define OPMX_MOE_MAX_EXPERTS_PER_TOKEN 32
@@ -126,21 +114,6 @@ int opmx_moe_row_parallel_linear(const void *X, const int64_t *expert_offset, co
                                  const void *B, int E, int64_t R, int64_t K, int64_t N,
                                  int dtype, int64_t rows_per_expert_hint,
                                  void *Y, void *workspace, size_t workspace_bytes, void *stream);
-
-/* The same grouped GEMM with the weight layout as an argument (opmx_weight_layout); the two
- * entry points above are this one with OPMX_WEIGHTS_ROW_MAJOR.  The reference has one weight
- * layout only (MoeColumnParallelLinear.py:66, MoeRowParallelLinear.py:52: F.linear on W[i]);
- * the tiled one is an offline repacking of the same values, made by opmx_moe_retile_weights when
- * the checkpoint is loaded (the step of Model.load_state_dict, Model.py:399-413). */
-int opmx_moe_grouped_linear(const void *X, const int64_t *expert_offset, const void *W, const void *B,
-                            int E, int64_t R, int64_t K, int64_t N, int dtype, int epilogue,
-                            int weight_layout, int64_t rows_per_expert_hint,
-                            void *Y, void *workspace, size_t workspace_bytes, void *stream);
-
-/* Copies W_in [E,N,K] into W_out in layout `to_layout`, from the other layout (W_in != W_out, no
- * overlap).  OPMX_ERR_UNSUPPORTED unless f16/bf16, N % 16 == 0 and K % 64 == 0. */
-int opmx_moe_retile_weights(const void *W_in, int E, int64_t N, int64_t K, int dtype, int to_layout,
-                            void *W_out, void *stream);
 
 /* SwiGLU.  Replaces SwiGLU.forward, torch_function/SwiGLU.py:11-17:
  *   Y[r, i] = X[r, D+i] * X[r, i] * sigmoid(beta * X[r, i]);  X [R,2D], Y [R,D]. */

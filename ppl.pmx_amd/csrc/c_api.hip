@@ -53,18 +53,14 @@ size_t grouped_gemm_workspace_bytes(int E, int64_t R, int64_t K, int64_t N, int 
 }
 
 int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
-                        int64_t K, int64_t N, int dtype, int epilogue, int weight_layout, int64_t rows_hint, void *Y,
-                        void *ws, size_t ws_bytes, hipStream_t s)
+                        int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint, void *Y, void *ws,
+                        size_t ws_bytes, hipStream_t s)
 {
     const int64_t ncols = epilogue == OPMX_EPILOGUE_SWIGLU ? N / 2 : N;
     if (R == 0 || ncols == 0) return OPMX_OK;
     const bool lowp = dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16;
-    const bool w_tiled = weight_layout == OPMX_WEIGHTS_TILED_16X64;
-    // what opmx_moe_retile_weights accepts, plus whole row groups per SwiGLU half
-    if (w_tiled && !(lowp && K % 64 == 0 && N % 16 == 0 && ncols % 16 == 0)) return OPMX_ERR_UNSUPPORTED;
     const bool mfma_ok = lowp && K > 0 && K % 8 == 0 && aligned16(X) && aligned16(W) &&
                          N * K < (int64_t{1} << 31) && R * K < (int64_t{1} << 40);
-    if (w_tiled && !mfma_ok) return OPMX_ERR_UNSUPPORTED;         // the generic kernel reads the reference layout only
     const bool tiled_ok = mfma_ok && K % 64 == 0;
     // Row-tile sizing: twice the mean rows per expert, never above what the caller can
     // guarantee.  An expert with more rows than one tile simply takes several tiles.
@@ -77,14 +73,14 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
     int choice;   // 1 generic, 2 tiled, 3 stream
     if (force == 3 && mfma_ok && stream_ws) choice = 3;
     else if (force == 2 && tiled_ok) choice = 2;
-    else if (force == 1 && !w_tiled) choice = 1;
+    else if (force == 1) choice = 1;
     else if (mfma_ok && stream_ws && hint <= kStreamMaxRowsPerExpert) choice = 3;
     else if (tiled_ok) choice = 2;
     else choice = 1;
 
     if (choice == 3)
         return launch_gemm_stream(X, off, W, B, E, R, K, N, dtype, epilogue, hint,
-                                  env_int("OPMX_MOE_GEMM_STREAM_VARIANT", 0), w_tiled, Y, s);
+                                  env_int("OPMX_MOE_GEMM_STREAM_VARIANT", 0), Y, s);
     if (choice == 2) {
         // Direct-to-LDS kernel from 128 mean rows per expert on, else 128x128 register-staged
         // (measured).  The direct-to-LDS kernel takes 256x256 tiles unless they would fill the CUs
@@ -94,7 +90,7 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
         const int64_t tiles256 = (R / 256 + (E + 1) / 2) * ((out_cols + 255) / 256);
         const int dflt = R / E >= 128 ? (tiles256 < 512 ? 3 : 0) : 2;
         return launch_gemm_tiled(X, off, W, B, E, R, K, N, dtype, epilogue,
-                                 env_int("OPMX_MOE_GEMM_TILED_VARIANT", dflt), w_tiled, Y, ws, ws_bytes, s);
+                                 env_int("OPMX_MOE_GEMM_TILED_VARIANT", dflt), Y, ws, ws_bytes, s);
     }
     return launch_gemm_generic(X, off, W, B, E, R, K, N, dtype, epilogue, Y, s);
 }
@@ -154,18 +150,16 @@ size_t opmx_moe_grouped_gemm_workspace_bytes(int E, int64_t R, int64_t K, int64_
 }
 
 static int grouped_checked(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
-                           int64_t K, int64_t N, int dtype, int epilogue, int weight_layout, int64_t hint, void *Y,
-                           void *ws, size_t ws_bytes, void *stream)
+                           int64_t K, int64_t N, int dtype, int epilogue, int64_t hint, void *Y, void *ws,
+                           size_t ws_bytes, void *stream)
 {
     if (E <= 0 || R < 0 || K < 0 || N < 0) return OPMX_ERR_BAD_ARGUMENT;
-    if (weight_layout != OPMX_WEIGHTS_ROW_MAJOR && weight_layout != OPMX_WEIGHTS_TILED_16X64) return OPMX_ERR_BAD_ARGUMENT;
     if (!dtype_ok(dtype) || E > OPMX_MOE_MAX_EXPERTS) return OPMX_ERR_UNSUPPORTED;
     if (epilogue != OPMX_EPILOGUE_NONE && epilogue != OPMX_EPILOGUE_SWIGLU) return OPMX_ERR_BAD_ARGUMENT;
     if (epilogue == OPMX_EPILOGUE_SWIGLU && N % 2) return OPMX_ERR_BAD_ARGUMENT;
     if (R == 0 || N == 0) return OPMX_OK;
     if (!X || !off || !W || !Y || K == 0) return OPMX_ERR_BAD_ARGUMENT;
-    return launch_grouped_gemm(X, off, W, B, E, R, K, N, dtype, epilogue, weight_layout, hint, Y, ws, ws_bytes,
-                               st(stream));
+    return launch_grouped_gemm(X, off, W, B, E, R, K, N, dtype, epilogue, hint, Y, ws, ws_bytes, st(stream));
 }
 
 int opmx_moe_column_parallel_linear(const void *X, const int64_t *expert_offset, const void *W, const void *B,
@@ -173,8 +167,8 @@ int opmx_moe_column_parallel_linear(const void *X, const int64_t *expert_offset,
                                     int64_t rows_per_expert_hint, void *Y, void *workspace,
                                     size_t workspace_bytes, void *stream)
 {
-    return grouped_checked(X, expert_offset, W, B, E, R, K, N, dtype, epilogue, OPMX_WEIGHTS_ROW_MAJOR,
-                           rows_per_expert_hint, Y, workspace, workspace_bytes, stream);
+    return grouped_checked(X, expert_offset, W, B, E, R, K, N, dtype, epilogue, rows_per_expert_hint, Y,
+                           workspace, workspace_bytes, stream);
 }
 
 int opmx_moe_row_parallel_linear(const void *X, const int64_t *expert_offset, const void *W, const void *B,
@@ -182,27 +176,8 @@ int opmx_moe_row_parallel_linear(const void *X, const int64_t *expert_offset, co
                                  int64_t rows_per_expert_hint, void *Y, void *workspace, size_t workspace_bytes,
                                  void *stream)
 {
-    return grouped_checked(X, expert_offset, W, B, E, R, K, N, dtype, OPMX_EPILOGUE_NONE, OPMX_WEIGHTS_ROW_MAJOR,
-                           rows_per_expert_hint, Y, workspace, workspace_bytes, stream);
-}
-
-int opmx_moe_grouped_linear(const void *X, const int64_t *expert_offset, const void *W, const void *B, int E,
-                            int64_t R, int64_t K, int64_t N, int dtype, int epilogue, int weight_layout,
-                            int64_t rows_per_expert_hint, void *Y, void *workspace, size_t workspace_bytes,
-                            void *stream)
-{
-    return grouped_checked(X, expert_offset, W, B, E, R, K, N, dtype, epilogue, weight_layout, rows_per_expert_hint,
+    return grouped_checked(X, expert_offset, W, B, E, R, K, N, dtype, OPMX_EPILOGUE_NONE, rows_per_expert_hint,
                            Y, workspace, workspace_bytes, stream);
-}
-
-int opmx_moe_retile_weights(const void *W_in, int E, int64_t N, int64_t K, int dtype, int to_layout, void *W_out,
-                            void *stream)
-{
-    if (E < 0 || N < 0 || K < 0) return OPMX_ERR_BAD_ARGUMENT;
-    if (to_layout != OPMX_WEIGHTS_ROW_MAJOR && to_layout != OPMX_WEIGHTS_TILED_16X64) return OPMX_ERR_BAD_ARGUMENT;
-    if (E == 0 || N == 0 || K == 0) return OPMX_OK;
-    if (!W_in || !W_out || W_in == W_out) return OPMX_ERR_BAD_ARGUMENT;
-    return launch_retile_weights(W_in, E, N, K, dtype, to_layout == OPMX_WEIGHTS_TILED_16X64, W_out, st(stream));
 }
 
 int opmx_swiglu(const void *X, int64_t R, int64_t D, float beta, int dtype, void *Y, void *stream)

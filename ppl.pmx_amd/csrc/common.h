@@ -84,14 +84,11 @@ int launch_swiglu(const void *X, int64_t R, int64_t D, float beta, int dtype, vo
 int launch_silu(const void *X, const void *gate, int64_t n, int dtype, void *Y, hipStream_t s);
 int launch_rms_norm(const void *X, const void *Wt, const void *Skip, int64_t T, int64_t H, float eps, int dtype,
                     void *Y, void *SkipOut, hipStream_t s);
-// to_tiled != 0: reference layout [E,N,K] -> 16x64 tiles (see weight_layout.hip); 0: back.  in != out.
-int launch_retile_weights(const void *in, int E, int64_t N, int64_t K, int dtype, int to_tiled, void *out,
-                          hipStream_t s);
 int launch_moe_reduce(const void *Y, const void *w, const int64_t *inv, int64_t T, int k, int64_t N,
                       int dtype, void *out, hipStream_t s);
 int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const void *B, int E,
-                        int64_t R, int64_t K, int64_t N, int dtype, int epilogue, int weight_layout,
-                        int64_t rows_hint, void *Y, void *ws, size_t ws_bytes, hipStream_t s);
+                        int64_t R, int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint,
+                        void *Y, void *ws, size_t ws_bytes, hipStream_t s);
 size_t grouped_gemm_workspace_bytes(int E, int64_t R, int64_t K, int64_t N, int dtype);
 
 }  // namespace opmx

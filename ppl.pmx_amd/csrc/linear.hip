@@ -111,7 +111,7 @@ int launch_linear(const void *X, const void *W, const void *B, int64_t T, int64_
     // reads X once with 128x128 tiles instead of one pass per 8 output features.
     if ((dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16) && T >= 512 && N > 8 && K % 64 == 0 &&
         aligned16(X) && aligned16(W) && N * K < (int64_t{1} << 31))
-        return launch_gemm_tiled(X, nullptr, W, B, 1, T, K, N, dtype, OPMX_EPILOGUE_NONE, /*128x128 tiles*/ 2, /*w_tiled*/ false, Y, nullptr, 0, s);
+        return launch_gemm_tiled(X, nullptr, W, B, 1, T, K, N, dtype, OPMX_EPILOGUE_NONE, /*128x128 tiles*/ 2, Y, nullptr, 0, s);
     switch (dtype) {
         case OPMX_DTYPE_F32: return linear_impl<float>(X, W, B, T, K, N, Y, s);
         case OPMX_DTYPE_F16: return linear_impl<f16>(X, W, B, T, K, N, Y, s);

@@ -144,14 +144,12 @@ int launch_gemm_generic(const void *X, const int64_t *off, const void *W, const 
 // 2 = 128x128 register-staged (4 waves).  off == nullptr: dense GEMM (one expert owns [0, R)).
 // ws / ws_bytes: optional scratch memory of gemm_tiled_workspace_bytes() bytes (variant 0 then
 // balances the last rounds of tiles over all CUs); nullptr / 0 is always accepted.
-// w_tiled: W is in the 16x64-tile layout of weight_layout.hip (needs 16 | N).
 int launch_gemm_tiled(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
-                      int64_t K, int64_t N, int dtype, int epilogue, int variant, bool w_tiled, void *Y, void *ws,
+                      int64_t K, int64_t N, int dtype, int epilogue, int variant, void *Y, void *ws,
                       size_t ws_bytes, hipStream_t s);
 size_t gemm_tiled_workspace_bytes();
-// w_tiled: W is in the 16x64-tile layout of weight_layout.hip (needs K % 64 == 0 and 16 | output columns).
 int launch_gemm_stream(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
-                       int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint, int variant, bool w_tiled,
-                       void *Y, hipStream_t s);
+                       int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint, int variant, void *Y,
+                       hipStream_t s);
 
 }  // namespace opmx

@@ -36,7 +36,7 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
                                                                const int64_t *__restrict__ off,
                                                                const T *__restrict__ W,
                                                                const T *__restrict__ Bias, int E, int64_t R,
-                                                               int64_t K, int64_t N, T *__restrict__ Y, int w_tiled)
+                                                               int64_t K, int64_t N, T *__restrict__ Y)
 {
     constexpr int NG = SG ? 2 : 1;               // row groups per wave: SwiGLU pairs gate rows with up rows
     constexpr int SROWS = 16 * SW;               // output columns per block
@@ -71,32 +71,17 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
     const char *xb = reinterpret_cast<const char *>(X + mt.row0 * K);
     const int wl_row = lane / (64 / RPL);               // row inside one wave load
     const int wl_k = (lane % (64 / RPL)) * 8;           // k offset inside the chunk
-    uint32_t wrow[NG][NLW];                             // byte offset of this lane's 16 bytes at chunk 0
+    uint32_t wrow[NG][NLW];                             // byte offset of the row start
     int wdst[NG][NLW];
-    int wk[NLW];                                        // ... and their k inside the chunk
-    // Reference layout: a chunk advances every row by KC*2 bytes.  Tiled layout (16 x 64 tiles, see
-    // weight_layout.hip): the wave's 16 rows x KC are KC/64 consecutive tiles, 32*KC contiguous
-    // bytes, and wave load i simply takes bytes [1024 i, 1024 (i+1)) of them.
-    const int64_t wstep = w_tiled ? KC * 32 : KC * 2;
 #pragma unroll
     for (int g = 0; g < NG; ++g)
 #pragma unroll
         for (int i = 0; i < NLW; ++i) {
-            if (w_tiled) {
-                // whole row groups only (16 | ND); a wave past the last one reads the last one again
-                const int64_t nb = ((nbase < ND ? nbase : ND - 16) + g * ND) >> 4;
-                const int o = i * 1024 + lane * 16, in_tile = o & 2047;
-                wk[i] = (o >> 11) * 64 + ((in_tile & 127) >> 1);
-                wrow[g][i] = static_cast<uint32_t>(nb * K * 32 + o);
-                wdst[g][i] = (g * 16 + (in_tile >> 7)) * RS + wk[i] * 2;
-            } else {
-                const int row = i * RPL + wl_row;
-                int64_t n = nbase + row;
-                n = (n < ND ? n : ND - 1) + g * ND;
-                wk[i] = wl_k;
-                wrow[g][i] = static_cast<uint32_t>(n * K * 2 + wl_k * 2);
-                wdst[g][i] = (g * 16 + row) * RS + wl_k * 2;
-            }
+            const int row = i * RPL + wl_row;
+            int64_t n = nbase + row;
+            n = (n < ND ? n : ND - 1) + g * ND;
+            wrow[g][i] = static_cast<uint32_t>(n * K * 2);
+            wdst[g][i] = (g * 16 + row) * RS + wl_k * 2;
         }
     uint32_t xrow[NLX];
     int xdst[NLX], xk[NLX];
@@ -132,19 +117,19 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
         const int seq_ = (KCI);                                                                        \
         const int kci_ = seq_ >= nchunks ? nchunks : (seq_ + rot >= nchunks ? seq_ + rot - nchunks : seq_ + rot); \
         if (kci_ < nfull) {                                                                            \
-            const char *wk_ = wb + static_cast<int64_t>(kci_) * wstep;                                 \
+            const char *wk_ = wb + static_cast<int64_t>(kci_) * (KC * 2);                              \
             const char *xk_ = xb + static_cast<int64_t>(kci_) * (KC * 2);                              \
             _Pragma("unroll") for (int g = 0; g < NG; ++g)                                             \
                 _Pragma("unroll") for (int i = 0; i < NLW; ++i)                                        \
-                    wreg[SET][g][i] = ld16<NT>(wk_ + wrow[g][i]);                                      \
+                    wreg[SET][g][i] = ld16<NT>(wk_ + (wrow[g][i] + static_cast<uint32_t>(wl_k * 2)));  \
             _Pragma("unroll") for (int i = 0; i < NLX; ++i)                                            \
                 xreg[SET][i] = ld16<false>(xk_ + (xrow[i] + static_cast<uint32_t>(xk[i] * 2)));        \
-        } else if (kci_ < nchunks) { /* ragged last chunk: lanes past K read chunk 0, get 0 */   \
+        } else if (kci_ < nchunks) { /* ragged last chunk: lanes past K read the row start, get 0 */   \
             const int64_t k0_ = static_cast<int64_t>(kci_) * KC;                                       \
             _Pragma("unroll") for (int g = 0; g < NG; ++g)                                             \
                 _Pragma("unroll") for (int i = 0; i < NLW; ++i) {                                      \
-                    const bool in_ = k0_ + wk[i] < K;                                                  \
-                    const u32x4 v_ = ld16<false>(wb + (in_ ? static_cast<int64_t>(kci_) * wstep : int64_t{0}) + wrow[g][i]); \
+                    const bool in_ = k0_ + wl_k < K;                                                   \
+                    const u32x4 v_ = ld16<false>(wb + (wrow[g][i] + (in_ ? static_cast<uint32_t>((k0_ + wl_k) * 2) : 0u))); \
                     wreg[SET][g][i] = in_ ? v_ : zero4;                                                \
                 }                                                                                      \
             _Pragma("unroll") for (int i = 0; i < NLX; ++i) {                                          \
@@ -219,7 +204,7 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
 
 template <typename T, int MT, int KC, int DEPTH, bool NT, int SW, bool SG>
 int stream_launch_sw(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
-                     int64_t N, void *Y, int w_tiled, hipStream_t s)
+                     int64_t N, void *Y, hipStream_t s)
 {
     constexpr int SROWS = 16 * SW;
     constexpr int RS = KC * 2 + 16;
@@ -234,20 +219,20 @@ int stream_launch_sw(const void *X, const int64_t *off, const void *W, const voi
     }
     dim3 grid(static_cast<unsigned>(ceil_div(SG ? N / 2 : N, SROWS)), static_cast<unsigned>(max_mtiles(R, E, 16 * MT)));
     kern<<<grid, SW * 64, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
-                                     static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), w_tiled);
+                                     static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y));
     OPMX_LAUNCH_CHECK();
     return OPMX_OK;
 }
 
 template <typename T, int MT, int KC, int DEPTH, bool NT, bool SG = false>
 int stream_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
-                  int64_t N, void *Y, int w_tiled, hipStream_t s)
+                  int64_t N, void *Y, hipStream_t s)
 {
     // at most min(R, E) experts are active: with 64-column blocks that is this many work items
     const int64_t items = ceil_div(SG ? N / 2 : N, 64) * (R < E ? R : E);
     if (MT <= 2 && items < 512)
-        return stream_launch_sw<T, MT, KC, DEPTH, NT, 1, SG>(X, off, W, B, E, R, K, N, Y, w_tiled, s);
-    return stream_launch_sw<T, MT, KC, DEPTH, NT, 4, SG>(X, off, W, B, E, R, K, N, Y, w_tiled, s);
+        return stream_launch_sw<T, MT, KC, DEPTH, NT, 1, SG>(X, off, W, B, E, R, K, N, Y, s);
+    return stream_launch_sw<T, MT, KC, DEPTH, NT, 4, SG>(X, off, W, B, E, R, K, N, Y, s);
 }
 
 // Row-tile height MT*16 from the rows-per-expert bound m; K-chunk width per height
@@ -256,38 +241,38 @@ int stream_launch(const void *X, const int64_t *off, const void *W, const void *
 // instance only serves single-token calls.
 template <typename T, int KC1, int KC2, int KC4, int KC8, int DEPTH, bool NT>
 int stream_pick_mt(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
-                   int64_t N, int64_t m, void *Y, int w_tiled, hipStream_t s)
+                   int64_t N, int64_t m, void *Y, hipStream_t s)
 {
-    if (m <= 2) return stream_launch<T, 1, KC1, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, w_tiled, s);
-    if (m <= 32) return stream_launch<T, 2, KC2, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, w_tiled, s);
-    if (m <= 64) return stream_launch<T, 4, KC4, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, w_tiled, s);
-    return stream_launch<T, 8, KC8, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, w_tiled, s);
+    if (m <= 2) return stream_launch<T, 1, KC1, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
+    if (m <= 32) return stream_launch<T, 2, KC2, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
+    if (m <= 64) return stream_launch<T, 4, KC4, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
+    return stream_launch<T, 8, KC8, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
 }
 
 // SwiGLU epilogue: a wave streams twice the rows, so the K chunks are half as wide.
 template <typename T>
 int stream_swiglu_impl(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
-                       int64_t N, int64_t rows_hint, void *Y, int w_tiled, hipStream_t s)
+                       int64_t N, int64_t rows_hint, void *Y, hipStream_t s)
 {
     const int64_t m = rows_hint > 0 ? rows_hint : R;
-    if (m <= 2) return stream_launch<T, 1, 256, 2, true, true>(X, off, W, B, E, R, K, N, Y, w_tiled, s);
-    if (m <= 32) return stream_launch<T, 2, 128, 2, true, true>(X, off, W, B, E, R, K, N, Y, w_tiled, s);
-    if (m <= 64) return stream_launch<T, 4, 64, 2, true, true>(X, off, W, B, E, R, K, N, Y, w_tiled, s);
-    return stream_launch<T, 8, 64, 2, true, true>(X, off, W, B, E, R, K, N, Y, w_tiled, s);
+    if (m <= 2) return stream_launch<T, 1, 256, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);
+    if (m <= 32) return stream_launch<T, 2, 128, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);
+    if (m <= 64) return stream_launch<T, 4, 64, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);
+    return stream_launch<T, 8, 64, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);
 }
 
 template <typename T>
 int stream_impl(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
-                int64_t N, int64_t rows_hint, int variant, void *Y, int w_tiled, hipStream_t s)
+                int64_t N, int64_t rows_hint, int variant, void *Y, hipStream_t s)
 {
     const int64_t m = rows_hint > 0 ? rows_hint : R;
     switch (variant) {   // tuning knob; every variant computes the same thing
-        case 1: return stream_pick_mt<T, 256, 256, 128, 128, 1, false>(X, off, W, B, E, R, K, N, m, Y, w_tiled, s);
-        case 2: return stream_pick_mt<T, 512, 512, 256, 128, 1, true>(X, off, W, B, E, R, K, N, m, Y, w_tiled, s);
-        case 3: return stream_pick_mt<T, 256, 256, 128, 64, 2, false>(X, off, W, B, E, R, K, N, m, Y, w_tiled, s);
-        case 4: return stream_pick_mt<T, 256, 128, 64, 64, 2, true>(X, off, W, B, E, R, K, N, m, Y, w_tiled, s);
-        case 5: return stream_pick_mt<T, 256, 256, 128, 128, 2, true>(X, off, W, B, E, R, K, N, m, Y, w_tiled, s);
-        default: return stream_pick_mt<T, 256, 256, 128, 64, 2, true>(X, off, W, B, E, R, K, N, m, Y, w_tiled, s);
+        case 1: return stream_pick_mt<T, 256, 256, 128, 128, 1, false>(X, off, W, B, E, R, K, N, m, Y, s);
+        case 2: return stream_pick_mt<T, 512, 512, 256, 128, 1, true>(X, off, W, B, E, R, K, N, m, Y, s);
+        case 3: return stream_pick_mt<T, 256, 256, 128, 64, 2, false>(X, off, W, B, E, R, K, N, m, Y, s);
+        case 4: return stream_pick_mt<T, 256, 128, 64, 64, 2, true>(X, off, W, B, E, R, K, N, m, Y, s);
+        case 5: return stream_pick_mt<T, 256, 256, 128, 128, 2, true>(X, off, W, B, E, R, K, N, m, Y, s);
+        default: return stream_pick_mt<T, 256, 256, 128, 64, 2, true>(X, off, W, B, E, R, K, N, m, Y, s);
     }
 }
 
@@ -295,20 +280,17 @@ int stream_impl(const void *X, const int64_t *off, const void *W, const void *B,
 
 // Requires: dtype f16/bf16, K % 8 == 0, 16-byte aligned X and W.
 int launch_gemm_stream(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
-                       int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint, int variant, bool w_tiled,
-                       void *Y, hipStream_t s)
+                       int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint, int variant, void *Y,
+                       hipStream_t s)
 {
-    const int64_t ncols = epilogue == OPMX_EPILOGUE_SWIGLU ? N / 2 : N;
-    if (w_tiled && (K % 64 != 0 || ncols % 16 != 0)) return OPMX_ERR_UNSUPPORTED;
-    const int wt = w_tiled ? 1 : 0;
     if (epilogue == OPMX_EPILOGUE_SWIGLU) {
-        if (dtype == OPMX_DTYPE_F16) return stream_swiglu_impl<f16>(X, off, W, B, E, R, K, N, rows_hint, Y, wt, s);
-        if (dtype == OPMX_DTYPE_BF16) return stream_swiglu_impl<bf16>(X, off, W, B, E, R, K, N, rows_hint, Y, wt, s);
+        if (dtype == OPMX_DTYPE_F16) return stream_swiglu_impl<f16>(X, off, W, B, E, R, K, N, rows_hint, Y, s);
+        if (dtype == OPMX_DTYPE_BF16) return stream_swiglu_impl<bf16>(X, off, W, B, E, R, K, N, rows_hint, Y, s);
         return OPMX_ERR_UNSUPPORTED;
     }
     switch (dtype) {
-        case OPMX_DTYPE_F16: return stream_impl<f16>(X, off, W, B, E, R, K, N, rows_hint, variant, Y, wt, s);
-        case OPMX_DTYPE_BF16: return stream_impl<bf16>(X, off, W, B, E, R, K, N, rows_hint, variant, Y, wt, s);
+        case OPMX_DTYPE_F16: return stream_impl<f16>(X, off, W, B, E, R, K, N, rows_hint, variant, Y, s);
+        case OPMX_DTYPE_BF16: return stream_impl<bf16>(X, off, W, B, E, R, K, N, rows_hint, variant, Y, s);
     }
     return OPMX_ERR_UNSUPPORTED;
 }

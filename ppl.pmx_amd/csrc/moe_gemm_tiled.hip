@@ -35,16 +35,6 @@ constexpr int CH = ROWB / 16;          // 16-byte chunks per row (8)
 // column land in sixteen different 16-byte bank groups (conflict-free b128 fragment reads).
 __device__ __forceinline__ int lds_off(int row, int chunk) { return row * ROWB + ((chunk ^ ((row >> 1) & 7)) << 4); }
 
-// Byte offset, from the start of W[e] at k-tile 0, of 16-byte chunk c8 (0..7) of the 64 k of row
-// `wrow`: reference layout [N,K] row-major, or the 16 x 64-tile layout of weight_layout.hip, in
-// which one k-tile further on is 2 KiB further on instead of 128 bytes.
-__device__ __forceinline__ uint32_t w_chunk_offset(int64_t wrow, int64_t K, int c8, int w_tiled)
-{
-    if (w_tiled) return static_cast<uint32_t>((wrow >> 4) * K * 32 + (wrow & 15) * 128 + c8 * 16);
-    return static_cast<uint32_t>((wrow * K + c8 * 8) * 2);
-}
-__device__ __forceinline__ int w_ktile_bytes(int w_tiled) { return w_tiled ? 2048 : ROWB; }
-
 // Clamped copy of expert_offset in LDS (values forced into a non-decreasing sequence inside
 // [0, R] when read, so a corrupt offset can never send a store outside Y).  Nothing to do for a
 // dense GEMM (off == nullptr).  Every thread must call it: it contains a block barrier.
@@ -422,7 +412,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
                                                                   const T *__restrict__ W,
                                                                   const T *__restrict__ Bias, int E, int64_t R,
                                                                   int64_t K, int64_t N, T *__restrict__ Y,
-                                                                  int ntiles_n, int gnx, int w_tiled)
+                                                                  int ntiles_n, int gnx)
 {
     constexpr int NT = WM * WN * 64;
     constexpr int WTM = BM / WM, WTN = BN / WN;          // wave tile: WTM X-rows x WTN W-rows
@@ -480,9 +470,8 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
         } else {
             wrow = n0 + row < N ? n0 + row : N - 1;
         }
-        b_src[i] = w_chunk_offset(wrow, K, sc, w_tiled);
+        b_src[i] = static_cast<uint32_t>((wrow * K + sc * 8) * 2);
     }
-    const int wkb = w_ktile_bytes(w_tiled);
 
     float4_t acc[TNS][TMS];
 #pragma unroll
@@ -517,8 +506,8 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
             rq[Q] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(Xt + ko_) +    \
                                                      a_src[(Q) < LA ? (Q) : 0]);                   \
         else                                                                                       \
-            rq[Q] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(We) +          \
-                                                     static_cast<int64_t>(KT) * wkb + b_src[(Q) < LA ? 0 : (Q)-LA]); \
+            rq[Q] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(We + ko_) +    \
+                                                     b_src[(Q) < LA ? 0 : (Q)-LA]);                \
     } while (0)
 #define OPMX_DRAINQ(Q, BUF)                                                                        \
     do {                                                                                           \
@@ -687,7 +676,7 @@ __device__ __forceinline__ void load_to_lds_16(__amdgpu_buffer_rsrc_t r, char *l
 // W-rows are WTN/2 gate rows followed by the WTN/2 up rows of the same output columns.
 template <int LA, int LB, int WTN, bool SWIGLU>
 __device__ __forceinline__ void tile_sources(int rows, int64_t n0, int64_t K, int64_t N, int64_t ncols, int wave,
-                                             int lane, int w_tiled, uint32_t (&a_src)[LA], uint32_t (&b_src)[LB])
+                                             int lane, uint32_t (&a_src)[LA], uint32_t (&b_src)[LB])
 {
     const int lrow8 = lane >> 3, slot = lane & 7;
 #pragma unroll
@@ -710,7 +699,7 @@ __device__ __forceinline__ void tile_sources(int rows, int64_t n0, int64_t K, in
             wrow = n0 + row < N ? n0 + row : N - 1;
         }
         const int c = slot ^ ((row >> 1) & 7);
-        b_src[i] = w_chunk_offset(wrow, K, c, w_tiled);
+        b_src[i] = static_cast<uint32_t>((wrow * K + c * 8) * 2);
     }
 }
 
@@ -780,8 +769,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
                                                                const T *__restrict__ Bias, int E, int64_t R,
                                                                int64_t K, int64_t N, T *__restrict__ Y,
                                                                int ntiles_n, int gnx, int sk_wgs, int sk_cost,
-                                                               float *__restrict__ sk_part, int *__restrict__ sk_count,
-                                                               int w_tiled)
+                                                               float *__restrict__ sk_part, int *__restrict__ sk_count)
 {
     constexpr int NW = 4, WM = BM / 128, WN = NW / WM;                 // 256 x 256: 2 x 2 waves, 128 x 256: 1 x 4
     constexpr int WTM = BM / WM, WTN = BN / WN, TMS = WTM / 16, TNS = WTN / 16, HM = TMS / 2;
@@ -842,9 +830,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
     const __amdgpu_buffer_rsrc_t rw = raw_descriptor(W + static_cast<int64_t>(mt.e) * N * K);
 
     uint32_t a_src[LA], b_src[LB];     // byte offsets from the tile's X / W base at k = 0
-    tile_sources<LA, LB, WTN, SWIGLU>(mt.rows, n0, K, N, ncols, wave, lane, w_tiled, a_src, b_src);
+    tile_sources<LA, LB, WTN, SWIGLU>(mt.rows, n0, K, N, ncols, wave, lane, a_src, b_src);
     const int a_lds = wave * LA * 1024, b_lds = BM * ROWB + wave * LB * 1024;   // wave-uniform
-    const int wkb = w_ktile_bytes(w_tiled);
 
     float4_t acc[TNS][TMS];
 #pragma unroll
@@ -865,8 +852,9 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
 #define OPMX_ISSUE1(KT, BUF, Q)                                                                    \
     do {                                                                                           \
         char *st_ = smem + (BUF)*STAGE;                                                            \
-        if ((Q) < LA) load_to_lds_16(rx, st_ + a_lds + (Q)*1024, a_src[(Q) < LA ? (Q) : 0], (KT)*ROWB); \
-        else load_to_lds_16(rw, st_ + b_lds + ((Q)-LA) * 1024, b_src[(Q) < LA ? 0 : (Q)-LA], (KT)*wkb); \
+        const int kb_ = (KT)*ROWB;                                                                 \
+        if ((Q) < LA) load_to_lds_16(rx, st_ + a_lds + (Q)*1024, a_src[(Q) < LA ? (Q) : 0], kb_);  \
+        else load_to_lds_16(rw, st_ + b_lds + ((Q)-LA) * 1024, b_src[(Q) < LA ? 0 : (Q)-LA], kb_); \
     } while (0)
 #define OPMX_XFRAG(BUF, S, H, I)                                                                   \
     xf[S][H][I] = *reinterpret_cast<const frag *>(smem + (BUF)*STAGE + ((S) ? co1 : co0) + x_off + ((H)*HM + (I)) * 16 * ROWB)
@@ -1131,8 +1119,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
                                                                        const T *__restrict__ W,
                                                                        const T *__restrict__ Bias, int E, int64_t R,
                                                                        int64_t K, int64_t N, T *__restrict__ Y,
-                                                                       int ntiles_n, int gnx, int sk_wgs, int sk_cost,
-                                                                       int w_tiled)
+                                                                       int ntiles_n, int gnx, int sk_wgs, int sk_cost)
 {
     constexpr int WM = 2, WN = 2, NW = 4;
     constexpr int WTM = BM / WM, WTN = BN / WN, TMS = WTM / 16, TNS = WTN / 16, HM = TMS / 2;
@@ -1176,9 +1163,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
     __amdgpu_buffer_rsrc_t rx = raw_descriptor(X + cur.row0 * K);
     __amdgpu_buffer_rsrc_t rw = raw_descriptor(W + static_cast<int64_t>(cur.e) * N * K);
     uint32_t a_src[LA], b_src[LB];
-    tile_sources<LA, LB, WTN, SWIGLU>(cur.rows, static_cast<int64_t>(cur_n) * BNO, K, N, ncols, wave, lane, w_tiled, a_src, b_src);
+    tile_sources<LA, LB, WTN, SWIGLU>(cur.rows, static_cast<int64_t>(cur_n) * BNO, K, N, ncols, wave, lane, a_src, b_src);
     const int a_lds = wave * LA * 1024, b_lds = BM * ROWB + wave * LB * 1024;
-    const int wkb = w_ktile_bytes(w_tiled);
     char *stg = smem + 2 * STAGE + wave * STG;
 
     float4_t acc[TNS][TMS];            // every tile's first k-tile defines all of them
@@ -1236,7 +1222,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
         // all loads of this tile are issued: retarget the load state, then stream on
         rx = raw_descriptor(X + nxt.row0 * K);
         rw = raw_descriptor(W + static_cast<int64_t>(nxt.e) * N * K);
-        tile_sources<LA, LB, WTN, SWIGLU>(nxt.rows, static_cast<int64_t>(nxt_n) * BNO, K, N, ncols, wave, lane, w_tiled, a_src, b_src);
+        tile_sources<LA, LB, WTN, SWIGLU>(nxt.rows, static_cast<int64_t>(nxt_n) * BNO, K, N, ncols, wave, lane, a_src, b_src);
         const int64_t nw0 = static_cast<int64_t>(cur_n) * BNO + wn * (SWIGLU ? WTN / 2 : WTN);   // first output column of this wave
         T bg[NOB][4], bu[NOB][4];          // bias of this lane's columns, requested ahead of the last loads
         if (BIAS) load_bias_regs<T, NOB, SWIGLU>(Bias + static_cast<int64_t>(cur.e) * N, ncols, nw0, lane, bg, bu);
@@ -1284,7 +1270,7 @@ __global__ void sk_clear_kernel(int *__restrict__ count, int n)
 
 template <typename T, int BM, int BN, int WM, int WN>
 int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
-                   int64_t N, int epilogue, void *Y, int w_tiled, hipStream_t s)
+                   int64_t N, int epilogue, void *Y, hipStream_t s)
 {
     constexpr int smem = 2 * (BM + BN) * ROWB;
     const bool sw = epilogue == OPMX_EPILOGUE_SWIGLU;
@@ -1305,7 +1291,7 @@ int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B
             attr_done[1] = true;
         }
         kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
-                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_n, gnx, w_tiled);
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_n, gnx);
     } else {
         auto kern = gemm_tiled_kernel<T, BM, BN, WM, WN, false>;
         if (!attr_done[0]) {
@@ -1315,7 +1301,7 @@ int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B
             attr_done[0] = true;
         }
         kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
-                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_n, gnx, w_tiled);
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_n, gnx);
     }
     OPMX_LAUNCH_CHECK();
     return OPMX_OK;
@@ -1346,8 +1332,7 @@ size_t sk_workspace_bytes(int cus)
 
 template <typename T, int BM, int BN>
 int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
-                      int64_t K, int64_t N, int epilogue, void *Y, void *ws, size_t ws_bytes, int w_tiled,
-                      hipStream_t s)
+                      int64_t K, int64_t N, int epilogue, void *Y, void *ws, size_t ws_bytes, hipStream_t s)
 {
     static_assert(BM * BN <= kSkTile, "tail slot size");
     constexpr int smem = 2 * (BM + BN) * ROWB;
@@ -1407,7 +1392,7 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
         static bool attr_p[4] = {false, false, false, false};
         const bool hb = B != nullptr;
         using kernel_t = void (*)(const T *, const int64_t *, const T *, const T *, int, int64_t, int64_t, int64_t, T *, int,
-                                  int, int, int, int);
+                                  int, int, int);
         const kernel_t kp = sw ? (hb ? gemm_tiled_dlds_persist_kernel<T, BM, BN, true, true>
                                      : gemm_tiled_dlds_persist_kernel<T, BM, BN, true, false>)
                                : (hb ? gemm_tiled_dlds_persist_kernel<T, BM, BN, false, true>
@@ -1422,14 +1407,14 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
         // ids congruent mod 8 stay on one XCD as long as the grid is a multiple of 8
         const unsigned wgs = static_cast<unsigned>(dp_ids < cus ? dp_ids : cus);
         if (sk_wgs > 0) sk_clear_kernel<<<1, 256, 0, s>>>(sk_count, kSkCounters);
-        kp<<<wgs, block, smem_p, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n, gnx, sk_wgs, sk_cost, w_tiled);
+        kp<<<wgs, block, smem_p, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n, gnx, sk_wgs, sk_cost);
         if (sk_wgs > 0) {
             if (sw)
                 gemm_tiled_dlds_kernel<T, BM, BN, true, true><<<sk_wgs, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
-                                                                                          gnx, sk_wgs, sk_cost, sk_part, sk_count, w_tiled);
+                                                                                          gnx, sk_wgs, sk_cost, sk_part, sk_count);
             else
                 gemm_tiled_dlds_kernel<T, BM, BN, false, true><<<sk_wgs, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
-                                                                                           gnx, sk_wgs, sk_cost, sk_part, sk_count, w_tiled);
+                                                                                           gnx, sk_wgs, sk_cost, sk_part, sk_count);
         }
         OPMX_LAUNCH_CHECK();
         return OPMX_OK;
@@ -1437,16 +1422,16 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
     if (sk_wgs > 0) sk_clear_kernel<<<1, 256, 0, s>>>(sk_count, kSkCounters);
     if (sw) {
         gemm_tiled_dlds_kernel<T, BM, BN, true, false><<<grid, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
-                                                                                 gnx, sk_wgs, sk_cost, sk_part, sk_count, w_tiled);
+                                                                                 gnx, sk_wgs, sk_cost, sk_part, sk_count);
         if (sk_wgs > 0)
             gemm_tiled_dlds_kernel<T, BM, BN, true, true><<<sk_wgs, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
-                                                                                      gnx, sk_wgs, sk_cost, sk_part, sk_count, w_tiled);
+                                                                                      gnx, sk_wgs, sk_cost, sk_part, sk_count);
     } else {
         gemm_tiled_dlds_kernel<T, BM, BN, false, false><<<grid, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
-                                                                                  gnx, sk_wgs, sk_cost, sk_part, sk_count, w_tiled);
+                                                                                  gnx, sk_wgs, sk_cost, sk_part, sk_count);
         if (sk_wgs > 0)
             gemm_tiled_dlds_kernel<T, BM, BN, false, true><<<sk_wgs, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
-                                                                                       gnx, sk_wgs, sk_cost, sk_part, sk_count, w_tiled);
+                                                                                       gnx, sk_wgs, sk_cost, sk_part, sk_count);
     }
     OPMX_LAUNCH_CHECK();
     return OPMX_OK;
@@ -1454,13 +1439,13 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
 
 template <typename T>
 int tiled_impl(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
-               int64_t N, int epilogue, int variant, void *Y, void *ws, size_t ws_bytes, int w_tiled, hipStream_t s)
+               int64_t N, int epilogue, int variant, void *Y, void *ws, size_t ws_bytes, hipStream_t s)
 {
     switch (variant) {
-        case 1: return tiled_launch<T, 256, 256, 2, 4>(X, off, W, B, E, R, K, N, epilogue, Y, w_tiled, s);
-        case 2: return tiled_launch<T, 128, 128, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, w_tiled, s);
-        case 3: return tiled_dlds_launch<T, 128, 256>(X, off, W, B, E, R, K, N, epilogue, Y, ws, ws_bytes, w_tiled, s);
-        default: return tiled_dlds_launch<T, 256, 256>(X, off, W, B, E, R, K, N, epilogue, Y, ws, ws_bytes, w_tiled, s);
+        case 1: return tiled_launch<T, 256, 256, 2, 4>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        case 2: return tiled_launch<T, 128, 128, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        case 3: return tiled_dlds_launch<T, 128, 256>(X, off, W, B, E, R, K, N, epilogue, Y, ws, ws_bytes, s);
+        default: return tiled_dlds_launch<T, 256, 256>(X, off, W, B, E, R, K, N, epilogue, Y, ws, ws_bytes, s);
     }
 }
 
@@ -1470,14 +1455,12 @@ int tiled_impl(const void *X, const int64_t *off, const void *W, const void *B, 
 // ws / ws_bytes: optional scratch memory (gemm_tiled_workspace_bytes()); with it the default
 // variant balances the last rounds of tiles over all CUs.
 int launch_gemm_tiled(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
-                      int64_t K, int64_t N, int dtype, int epilogue, int variant, bool w_tiled, void *Y, void *ws,
+                      int64_t K, int64_t N, int dtype, int epilogue, int variant, void *Y, void *ws,
                       size_t ws_bytes, hipStream_t s)
 {
-    if (w_tiled && N % 16 != 0) return OPMX_ERR_UNSUPPORTED;      // K % 64 == 0 is required anyway
-    const int wt = w_tiled ? 1 : 0;
     switch (dtype) {
-        case OPMX_DTYPE_F16: return tiled_impl<f16>(X, off, W, B, E, R, K, N, epilogue, variant, Y, ws, ws_bytes, wt, s);
-        case OPMX_DTYPE_BF16: return tiled_impl<bf16>(X, off, W, B, E, R, K, N, epilogue, variant, Y, ws, ws_bytes, wt, s);
+        case OPMX_DTYPE_F16: return tiled_impl<f16>(X, off, W, B, E, R, K, N, epilogue, variant, Y, ws, ws_bytes, s);
+        case OPMX_DTYPE_BF16: return tiled_impl<bf16>(X, off, W, B, E, R, K, N, epilogue, variant, Y, ws, ws_bytes, s);
     }
     return OPMX_ERR_UNSUPPORTED;
 }

@@ -33,19 +33,6 @@ class _MoeLinearBase(nn.Module):
             self.bias = nn.Parameter(torch.zeros(*b_shape, **kw), requires_grad=False)
         else:
             self.register_parameter("bias", None)
-        self.weight_layout = OPMX.WEIGHTS_ROW_MAJOR
-
-    @torch.no_grad()
-    def retile_(self, layout=None):
-        """Repacks ``weight`` in place of the old storage into ``layout`` (default: the 16x64-tile
-        layout the streaming kernels read 7-9 % faster; ``OPMX.WEIGHTS_ROW_MAJOR`` goes back).
-        An addition to the reference's module: do it once after loading.  ``state_dict`` and ONNX
-        export see the bytes as they are, so go back to row-major before saving or exporting."""
-        layout = OPMX.WEIGHTS_TILED_16X64 if layout is None else layout
-        if layout != self.weight_layout:
-            self.weight.data = OPMX.moe_retile_weights(self.weight.data, layout)
-            self.weight_layout = layout
-        return self
 
 
 class MoeColumnParallelLinear(_MoeLinearBase):
@@ -60,10 +47,9 @@ class MoeColumnParallelLinear(_MoeLinearBase):
         self.gather_output = gather_output
 
     def forward(self, X: torch.Tensor, expert_offset: torch.Tensor):
-        op = OPMX.moe_column_parallel_linear if self.weight_layout == OPMX.WEIGHTS_ROW_MAJOR \
-            else OPMX.moe_column_parallel_linear_tiled
-        return op(X, expert_offset, self.weight, self.bias, self.proc_group, self.num_experts, self.in_features,
-                  self.out_features, self.gather_output)
+        return OPMX.moe_column_parallel_linear(X, expert_offset, self.weight, self.bias, self.proc_group,
+                                               self.num_experts, self.in_features, self.out_features,
+                                               self.gather_output)
 
 
 class MoeRowParallelLinear(_MoeLinearBase):
@@ -79,7 +65,6 @@ class MoeRowParallelLinear(_MoeLinearBase):
         self.input_is_parallel = input_is_parallel
 
     def forward(self, X: torch.Tensor, expert_offset: torch.Tensor):
-        op = OPMX.moe_row_parallel_linear if self.weight_layout == OPMX.WEIGHTS_ROW_MAJOR \
-            else OPMX.moe_row_parallel_linear_tiled
-        return op(X, expert_offset, self.weight, self.bias, self.proc_group, self.num_experts, self.in_features,
-                  self.out_features, self.input_is_parallel)
+        return OPMX.moe_row_parallel_linear(X, expert_offset, self.weight, self.bias, self.proc_group,
+                                            self.num_experts, self.in_features, self.out_features,
+                                            self.input_is_parallel)

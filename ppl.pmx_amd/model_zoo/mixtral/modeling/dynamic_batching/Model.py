@@ -69,21 +69,13 @@ class MoeFeedForward(nn.Module):
             if self.fuse_swiglu_epilogue and not torch.onnx.is_in_onnx_export():
                 x13 = OPMX.moe_column_parallel_linear_swiglu(
                     x_experts, expert_offset, self.wu.weight, self.wu.bias, self.num_experts,
-                    self.wu.in_features, self.wu.out_features, self.wu.weight_layout)
+                    self.wu.in_features, self.wu.out_features)
             else:
                 x13 = OPMX.swiglu(self.wu(x_experts, expert_offset))
         else:
             x13 = OPMX.silu(self.w1(x_experts, expert_offset), self.w3(x_experts, expert_offset))
         x_out = self.w2(x13, expert_offset)
         return OPMX.moe_reduce(x_out, expert_weights, invert_permutation, k)
-
-    def retile_(self, layout=None):
-        """Repacks the expert weights (``wu`` or ``w1``/``w3``, and ``w2``) for the streaming kernels,
-        see ``MoeColumnParallelLinear.retile_``; the router gate stays as it is."""
-        for name in ("wu", "w1", "w3", "w2"):
-            if hasattr(self, name):
-                getattr(self, name).retile_(layout)
-        return self
 
     @torch.no_grad()
     def load_state_dict(self, state_dict, strict: bool = True, prefix=None):
@@ -97,10 +89,6 @@ class MoeFeedForward(nn.Module):
         ``strict`` raises on a parameter left without a value or a shape mismatch.
         """
         prefix = "layers.{}.feed_forward.".format(self.layer_id) if prefix is None else prefix
-        for name in ("wu", "w1", "w3", "w2"):
-            if hasattr(self, name) and getattr(self, name).weight_layout != OPMX.WEIGHTS_ROW_MAJOR:
-                raise RuntimeError("load_state_dict: {} holds repacked weights; checkpoints are in the reference "
-                                   "layout, so load first and call retile_() afterwards".format(name))
         params = dict(self.named_parameters())
         used, filled = [], set()
 
@@ -138,7 +126,7 @@ class MoeFeedForward(nn.Module):
 
 
 def load_opmx_moe_block(path, layer_id: int, num_experts_per_token: int, fused_ffn_glu: bool = True,
-                        dtype=None, device=None, fuse_swiglu_epilogue: bool = False, retile: bool = False):
+                        dtype=None, device=None, fuse_swiglu_epilogue: bool = False):
     """Builds the MoE block of layer ``layer_id`` from an OPMX Mixtral ``.pth`` checkpoint.
 
     The file is opened with ``weights_only=True`` and memory-mapped, so only this layer's tensors are
@@ -155,6 +143,4 @@ def load_opmx_moe_block(path, layer_id: int, num_experts_per_token: int, fused_f
                            bias, None, dtype=gate.dtype if dtype is None else dtype, device=device,
                            fuse_swiglu_epilogue=fuse_swiglu_epilogue)
     block.load_state_dict(sd)
-    if retile:          # GPU only: repack the expert weights for the streaming kernels
-        block.retile_()
     return block

@@ -41,24 +41,11 @@ def moe_column_parallel_linear(X, expert_offset, W, B, proc_group, num_experts: 
 
 
 def moe_column_parallel_linear_swiglu(X, expert_offset, W, B, num_experts: int, in_features: int,
-                                      out_features: int, weight_layout: int = _lib.WEIGHTS_ROW_MAJOR) -> torch.Tensor:
+                                      out_features: int) -> torch.Tensor:
     """Fused form of ``swiglu(moe_column_parallel_linear(...))`` for the fused
     gate/up weight ``wu = [w1; w3]``: SwiGLU (beta = 1) is applied to the fp32
     accumulators, the [R, 2I] intermediate never reaches memory in the MFMA
     kernels.  No counterpart operator in the reference (it is the composition
     of ``Model.py:198`` and ``Model.py:200``); eager only."""
     assert X.shape[-1] == in_features, "X.shape is {}, in_features is {}".format(X.shape, in_features)
-    return grouped_linear("column", X, expert_offset, W, B, num_experts, epilogue=_lib.EPILOGUE_SWIGLU,
-                          weight_layout=weight_layout)
-
-
-def moe_column_parallel_linear_tiled(X, expert_offset, W, B, proc_group, num_experts: int, in_features: int,
-                                     out_features: int, gather_output: bool = True) -> torch.Tensor:
-    """``moe_column_parallel_linear`` for weights repacked by ``moe_retile_weights`` (same
-    arguments and result; eager only: an exported graph carries reference-layout weights)."""
-    assert X.shape[-1] == in_features, "X.shape is {}, in_features is {}".format(X.shape, in_features)
-    if torch.onnx.is_in_onnx_export():
-        raise RuntimeError("moe_column_parallel_linear_tiled: export needs the weights in the reference layout")
-    if _lib.world_size(proc_group) > 1:
-        raise NotImplementedError("moe_column_parallel_linear_tiled: this build covers one GPU, TP=1")
-    return grouped_linear("column", X, expert_offset, W, B, num_experts, weight_layout=_lib.WEIGHTS_TILED_16X64)
+    return grouped_linear("column", X, expert_offset, W, B, num_experts, epilogue=_lib.EPILOGUE_SWIGLU)

@@ -35,14 +35,3 @@ def moe_row_parallel_linear(X, expert_offset, W, B, proc_group, num_experts: int
                             out_features: int, input_is_parallel: bool = False):
     return MoeRowParallelLinear.apply(X, expert_offset, W, B, proc_group, num_experts, in_features,
                                       out_features, input_is_parallel)
-
-
-def moe_row_parallel_linear_tiled(X, expert_offset, W, B, proc_group, num_experts: int, in_features: int,
-                                  out_features: int, input_is_parallel: bool = False):
-    """``moe_row_parallel_linear`` for weights repacked by ``moe_retile_weights`` (same arguments
-    and result; eager only: an exported graph carries reference-layout weights)."""
-    if torch.onnx.is_in_onnx_export():
-        raise RuntimeError("moe_row_parallel_linear_tiled: export needs the weights in the reference layout")
-    if _lib.world_size(proc_group) > 1:
-        raise NotImplementedError("moe_row_parallel_linear_tiled: this build covers one GPU, TP=1")
-    return grouped_linear("row", X, expert_offset, W, B, num_experts, weight_layout=_lib.WEIGHTS_TILED_16X64)

@@ -4,16 +4,13 @@ import torch
 from . import _lib
 
 
-def grouped_linear(op, X, expert_offset, W, B, num_experts, epilogue=_lib.EPILOGUE_NONE,
-                   weight_layout=_lib.WEIGHTS_ROW_MAJOR):
+def grouped_linear(op, X, expert_offset, W, B, num_experts, epilogue=_lib.EPILOGUE_NONE):
     """``Y[off[e]:off[e+1]] = X[off[e]:off[e+1]] @ W[e]^T (+ B[e])`` on the GPU.
 
     ``op`` is "column" or "row".  Output dtype is ``W.dtype`` on ``X.device``
     (the reference's export branch states that dtype,
     ``MoeColumnParallelLinear.py:45``; its eager branch follows the process
     default dtype).  A row-parallel bias is applied per expert segment.
-    ``weight_layout``: how the values of ``W`` lie in memory (``W.shape`` is
-    ``[E, N, K]`` either way), see ``retile_weights``.
     """
     name = "moe_{}_parallel_linear".format(op)
     dev = _lib.require_gpu(name, X, expert_offset, W, B)
@@ -47,11 +44,7 @@ def grouped_linear(op, X, expert_offset, W, B, num_experts, epilogue=_lib.EPILOG
         ws = _lib.workspace(ws_bytes, dev)
     else:
         ws_bytes = 0
-    if weight_layout != _lib.WEIGHTS_ROW_MAJOR:
-        rc = L.opmx_moe_grouped_linear(_lib.ptr(Xf), _lib.ptr(off), _lib.ptr(Wc), _lib.ptr(Bc), E, R, K, N, dt,
-                                       epilogue, weight_layout, hint, _lib.ptr(Y), _lib.ptr(ws), ws_bytes,
-                                       _lib.stream_ptr(dev))
-    elif op == "column":
+    if op == "column":
         rc = L.opmx_moe_column_parallel_linear(_lib.ptr(Xf), _lib.ptr(off), _lib.ptr(Wc), _lib.ptr(Bc), E, R, K, N,
                                                dt, epilogue, hint, _lib.ptr(Y), _lib.ptr(ws), ws_bytes,
                                                _lib.stream_ptr(dev))
@@ -68,24 +61,3 @@ def linear_attrs(num_experts, in_features, out_features, has_bias, **extra):
                  bias_term_i=bool(has_bias))
     attrs.update(extra)
     return attrs
-
-
-def retile_weights(W, to_layout=_lib.WEIGHTS_TILED_16X64):
-    """A copy of the expert weights ``W [E, N, K]`` (fp16/bf16, on the GPU) in another memory layout.
-
-    ``WEIGHTS_TILED_16X64``: 16-row x 64-k tiles stored one after the other, in which the 16 weight
-    rows a wave streams are one contiguous run (+7-9 % decode bandwidth); ``WEIGHTS_ROW_MAJOR``: back
-    to the reference's row-major ``[N, K]`` per expert.  The input must be in the other layout; the
-    result has the same shape and dtype.  Needs ``N % 16 == 0`` and ``K % 64 == 0``.  Repacking is
-    what ``Model.load_state_dict`` (``Model.py:399-413`` of the reference) would do once per load.
-    """
-    dev = _lib.require_gpu("moe_retile_weights", W)
-    if W.dim() != 3:
-        raise ValueError("moe_retile_weights: W must be [num_experts, out_features, in_features]")
-    E, N, K = W.shape
-    dt = _lib.dtype_id(W, "moe_retile_weights")
-    Wc = W.detach().contiguous()
-    out = torch.empty_like(Wc)
-    rc = _lib.lib().opmx_moe_retile_weights(_lib.ptr(Wc), E, N, K, dt, to_layout, _lib.ptr(out), _lib.stream_ptr(dev))
-    _lib.check(rc, "moe_retile_weights")
-    return out

@@ -19,7 +19,6 @@ ABI_VERSION = 1
 
 F32, F16, BF16 = 0, 1, 2
 EPILOGUE_NONE, EPILOGUE_SWIGLU = 0, 1
-WEIGHTS_ROW_MAJOR, WEIGHTS_TILED_16X64 = 0, 1     # opmx_weight_layout
 MAX_EXPERTS, MAX_EXPERTS_PER_TOKEN = 256, 32
 
 _DTYPES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
@@ -37,9 +36,6 @@ _SIGNATURES = {
                                                _vp, _vp, _sz, _vp]),
     "opmx_moe_row_parallel_linear": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _i64,
                                             _vp, _vp, _sz, _vp]),
-    "opmx_moe_grouped_linear": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _int, _int, _i64,
-                                       _vp, _vp, _sz, _vp]),
-    "opmx_moe_retile_weights": (_int, [_vp, _int, _i64, _i64, _int, _int, _vp, _vp]),
     "opmx_swiglu": (_int, [_vp, _i64, _i64, _f, _int, _vp, _vp]),
     "opmx_silu": (_int, [_vp, _vp, _i64, _int, _vp, _vp]),
     "opmx_rms_norm": (_int, [_vp, _vp, _vp, _i64, _i64, _f, _int, _vp, _vp, _vp]),

@@ -222,94 +222,3 @@ def test_argument_errors():
         OPMX.moe_row_parallel_linear(X.cpu(), off.cpu(), W.cpu(), None, None, 1, 64, 32, True)
     Y = OPMX.moe_row_parallel_linear(X[:0], torch.zeros(2, dtype=torch.int64, device=d), W, None, None, 1, 64, 32)
     assert Y.shape == (0, 2, 32)
-
-
-def tiled(W):
-    """W [E,N,K] repacked into 16-row x 64-k tiles with torch alone (the definition of the layout)."""
-    E, N, K = W.shape
-    return W.view(E, N // 16, 16, K // 64, 64).permute(0, 1, 3, 2, 4).contiguous().view(E, N, K)
-
-
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_retile_weights_round_trip(dtype):
-    OPMX = opmx()
-    g = torch.Generator().manual_seed(5)
-    for E, N, K in ((3, 48, 192), (8, 4096, 1408 - 1408 % 64), (1, 16, 64)):
-        W = torch.randn(E, N, K, generator=g).to(dtype).to(dev())
-        T = OPMX.moe_retile_weights(W, OPMX.WEIGHTS_TILED_16X64)
-        assert T.shape == W.shape and T.dtype == W.dtype and torch.equal(T, tiled(W))
-        assert torch.equal(OPMX.moe_retile_weights(T, OPMX.WEIGHTS_ROW_MAJOR), W)
-    with pytest.raises(RuntimeError):
-        OPMX.moe_retile_weights(torch.zeros(2, 24, 64, dtype=dtype, device=dev()))       # N % 16
-    with pytest.raises(RuntimeError):
-        OPMX.moe_retile_weights(torch.zeros(2, 32, 96, dtype=dtype, device=dev()))       # K % 64
-
-
-TILED_W_CASES = [
-    # kernel family, env, sizes, K, N, bias, swiglu
-    ("stream", {"OPMX_MOE_GEMM": "stream"}, RAGGED8, 256, 96, True, False),
-    ("stream", {"OPMX_MOE_GEMM": "stream"}, RAGGED8, 4096, 1024, False, False),
-    ("stream ragged K chunk", {"OPMX_MOE_GEMM": "stream"}, [3, 0, 9, 1], 1408, 208, True, False),   # 16 | N, not 64
-    ("stream swiglu", {"OPMX_MOE_GEMM": "stream"}, RAGGED8, 512, 2 * 176, True, True),
-    ("stream 1 wave", {"OPMX_MOE_GEMM": "stream"}, [1, 0, 1, 0], 320, 64, False, False),
-    ("stream tall", {"OPMX_MOE_GEMM": "stream"}, [70, 3, 100, 40], 192, 128, False, True),
-    ("128x128", {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": "2"}, [300, 0, 129, 1, 256, 77, 0, 513], 192, 528, True, False),
-    ("128x128 swiglu", {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": "2"}, [300, 0, 129, 77], 128, 2 * 400, False, True),
-    ("256x256 reg", {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": "1"}, [300, 0, 129, 513], 128, 1040, True, False),
-    ("256x256 dlds", {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": "0", "OPMX_MOE_GEMM_PERSIST": "0"}, [300, 0, 129, 1, 256, 77, 0, 513], 192, 528, True, False),
-    ("256x256 persistent", {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": "0"}, [1500, 0, 700, 33, 1281, 256, 5, 1300], 320, 4096, True, False),
-    ("256x256 persistent swiglu", {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": "0"}, [1500, 0, 700, 33, 1281, 256, 5, 1300], 256, 4096, False, True),
-    ("256x256 tail split", {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": "0", "OPMX_MOE_GEMM_STREAMK": "2"}, [300, 77, 129], 2048, 4096, True, False),
-    ("128x256", {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": "3"}, [300, 0, 129, 513], 256, 2816, False, False),
-]
-
-
-@pytest.mark.parametrize("case", TILED_W_CASES, ids=[c[0] for c in TILED_W_CASES])
-def test_tiled_weight_layout_gives_the_same_bits(case):
-    """Every grouped-GEMM kernel reads the repacked weights: same result, bit for bit, as with the
-    reference layout (the accumulation order does not depend on where the weights lie)."""
-    _, env, sizes, K, N, bias, swiglu = case
-    OPMX = opmx()
-    dtype = torch.float16
-    E, R = len(sizes), sum(sizes)
-    g = torch.Generator().manual_seed(K + N + R)
-    X = torch.randn(R, K, generator=g).to(dtype).to(dev())
-    W = (torch.randn(E, N, K, generator=g) * 0.05).to(dtype).to(dev())
-    B = torch.randn(E, N, generator=g).to(dtype).to(dev()) if bias else None
-    off = offsets(sizes).to(dev())
-    Wt = OPMX.moe_retile_weights(W)
-    old = {k: os.environ.get(k) for k in env}
-    os.environ.update(env)
-    try:
-        if swiglu:
-            a = OPMX.moe_column_parallel_linear_swiglu(X, off, W, B, E, K, N)
-            b = OPMX.moe_column_parallel_linear_swiglu(X, off, Wt, B, E, K, N, OPMX.WEIGHTS_TILED_16X64)
-        else:
-            a = OPMX.moe_row_parallel_linear(X, off, W, B, None, E, K, N, True)
-            b = OPMX.moe_row_parallel_linear_tiled(X, off, Wt, B, None, E, K, N, True)
-        torch.cuda.synchronize()
-    finally:
-        for k, v in old.items():
-            if v is None:
-                os.environ.pop(k, None)
-            else:
-                os.environ[k] = v
-    ref = O.moe_column_parallel_linear(X.cpu(), off.cpu(), W.cpu(), None if B is None else B.cpu(), acc=torch.float64,
-                                       out_dtype=torch.float64)
-    if swiglu:
-        ref = O.swiglu(ref, acc=torch.float64)
-    assert_close_ulp(a, ref, dtype, ulps=2, floor=0.02, what=case[0])
-    assert torch.equal(a, b), case[0]
-
-
-def test_tiled_weight_layout_errors():
-    OPMX = opmx()
-    X = torch.zeros(4, 72, dtype=torch.float16, device=dev())
-    W = torch.zeros(2, 32, 72, dtype=torch.float16, device=dev())
-    off = torch.tensor([0, 2, 4], device=dev())
-    with pytest.raises(RuntimeError):      # K % 64 != 0 cannot be a repacked tensor
-        OPMX.moe_row_parallel_linear_tiled(X, off, W, None, None, 2, 72, 32, True)
-    Xf = torch.zeros(4, 64, dtype=torch.float32, device=dev())
-    Wf = torch.zeros(2, 32, 64, dtype=torch.float32, device=dev())
-    with pytest.raises(RuntimeError):      # fp32 has no repacked form
-        OPMX.moe_row_parallel_linear_tiled(Xf, off, Wf, None, None, 2, 64, 32, True)

@@ -46,10 +46,6 @@ def test_no_cpu_fallback():
         OPMX.linear(x, torch.randn(8, 16), None, 16, 8)
     with pytest.raises(RuntimeError, match="no CPU path"):
         OPMX.skip_rms_norm(x, torch.ones(16), x)
-    with pytest.raises(RuntimeError, match="no CPU path"):
-        OPMX.moe_retile_weights(torch.zeros(2, 16, 64, dtype=torch.float16))
-    with pytest.raises(RuntimeError, match="no CPU path"):
-        OPMX.moe_row_parallel_linear_tiled(x, torch.arange(3), torch.randn(2, 8, 16), None, None, 2, 16, 8, True)
     with pytest.raises(AssertionError):          # the reference's in_features assert comes first
         OPMX.moe_column_parallel_linear(x, torch.arange(3), torch.randn(2, 8, 16), None, None, 2, 15, 8, False)
 
@@ -134,23 +130,6 @@ def test_export_placeholders_have_eager_order_and_types():
     assert off.shape == (9,) and off.dtype == torch.int64
     text = str(graph)
     assert re.search(r"Half\(.*\), %\d+ : Half\(.*\), %\d+ : Long\(.*\), %\d+ : Long\(.*\) = opmx::MoeSelect", text)
-
-
-def test_repacked_weights_are_a_module_state():
-    """The layout travels with the module (not the tensor), checkpoints are reference layout."""
-    from model_zoo.ModelParallel import MoeColumnParallelLinear
-    from model_zoo.mixtral.modeling.dynamic_batching.Model import MoeFeedForward
-    sig = lambda f: list(inspect.signature(f).parameters)
-    assert sig(OPMX.moe_column_parallel_linear_tiled) == sig(OPMX.moe_column_parallel_linear)
-    assert sig(OPMX.moe_row_parallel_linear_tiled) == sig(OPMX.moe_row_parallel_linear)
-    m = MoeColumnParallelLinear(None, 2, 64, 32, bias_term=False, dtype=torch.float16)
-    assert m.weight_layout == OPMX.WEIGHTS_ROW_MAJOR and m.retile_(OPMX.WEIGHTS_ROW_MAJOR) is m   # no-op, no GPU needed
-    with pytest.raises(RuntimeError, match="no CPU path"):
-        m.retile_()
-    block = MoeFeedForward(MoeFeedForward.params(64, 32, 2, 1), 0, True, False, None, dtype=torch.float16)
-    block.wu.weight_layout = OPMX.WEIGHTS_TILED_16X64          # as retile_() leaves it
-    with pytest.raises(RuntimeError, match="reference layout"):
-        block.load_state_dict({})
 
 
 def test_tensor_parallel_is_refused():
