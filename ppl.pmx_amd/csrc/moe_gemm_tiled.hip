@@ -703,6 +703,15 @@ __device__ __forceinline__ void tile_sources(int rows, int64_t n0, int64_t K, in
     }
 }
 
+// Where a workgroup starts its walk over the nk k-tiles (it wraps around): an eighth of K further
+// on for every XCD.  The workgroups of one XCD keep walking together, which is what lets them
+// share operand tiles in their L2, but the XCDs no longer ask the memory for the same k offset
+// of every row at the same moment (rows lie a multiple of 8 KiB apart: such requests crowd onto
+// few channels).  Down projection (K = 14336) +2.5 %, K = 4096 ... 6144 +0.6 ... 1 %; not worth it
+// below 64 k-tiles.  The fp32 accumulation order then depends on the XCD, i.e. on the tile's
+// position in the launch: fixed for a given problem shape.
+__device__ __forceinline__ int k_rotation(int nk) { return nk >= 64 ? static_cast<int>(blockIdx.x & 7) * nk / 8 : 0; }
+
 // Tail balancing ("split-K of the last round").  With G workgroup slots (one per CU) the last
 // ttot % G tiles of the row-major tile order would run alone on a mostly idle chip.  When the
 // caller lends scratch memory they are left to a second launch in which each of them is cut
@@ -791,6 +800,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
     stage_offsets(off, E, R, s_off);
     const int mtiles = count_mtiles(off != nullptr, s_off, E, R, BM);
     const int nk = static_cast<int>(K / BK);
+    const int krot = k_rotation(nk);
     const int64_t ttot = static_cast<int64_t>(mtiles) * ntiles_n;
     const int g = sk_split(ttot, sk_wgs, nk, gnx, sk_cost);
     const int64_t tail = g > 1 ? ttot % sk_wgs : 0;      // tiles left to the tail launch
@@ -852,7 +862,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
 #define OPMX_ISSUE1(KT, BUF, Q)                                                                    \
     do {                                                                                           \
         char *st_ = smem + (BUF)*STAGE;                                                            \
-        const int kb_ = (KT)*ROWB;                                                                 \
+        const int kr_ = (KT) + krot;                     /* rotated k-tile, see k_rotation */       \
+        const int kb_ = (kr_ >= nk ? kr_ - nk : kr_) * ROWB;                                       \
         if ((Q) < LA) load_to_lds_16(rx, st_ + a_lds + (Q)*1024, a_src[(Q) < LA ? (Q) : 0], kb_);  \
         else load_to_lds_16(rw, st_ + b_lds + ((Q)-LA) * 1024, b_src[(Q) < LA ? 0 : (Q)-LA], kb_); \
     } while (0)
@@ -1143,6 +1154,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
     stage_offsets(off, E, R, s_off);
     const int mtiles = count_mtiles(off != nullptr, s_off, E, R, BM);
     const int nk = static_cast<int>(K / BK);
+    const int krot = k_rotation(nk);
     const int64_t ttot = static_cast<int64_t>(mtiles) * ntiles_n;
     const int g = sk_split(ttot, sk_wgs, nk, gnx, sk_cost);
     // ids [nmain, ttot) are the tail launch's.  The row-partition order has ids that name no tile
