@@ -184,6 +184,10 @@ def test_stream_kernel_variants(variant, dtype):
     # many weight rows: 4-wave blocks (the small cases above run the 1-wave blocks), ragged last slab
     run_case("column", [8, 9, 7, 11, 0, 16, 5, 8], 256, 4200, dtype, True, env)
     run_case("row", [30, 2, 17, 0, 32, 1, 25, 21], 512, 4160, dtype, False, env)
+    # 16 and more K chunks: every block starts its walk over K somewhere else and wraps around,
+    # also through a ragged last chunk and in the SwiGLU form
+    run_case("row", [8, 9, 7, 11, 0, 16, 5, 8], 8192 + 72, 320, dtype, True, env)
+    run_case("column", [30, 2, 17, 0, 32, 1, 25, 21], 4096, 2 * 192, dtype, False, env, swiglu=True)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
