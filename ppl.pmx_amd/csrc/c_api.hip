@@ -15,7 +15,7 @@ inline size_t elt(int d) { return d == OPMX_DTYPE_F32 ? 4 : 2; }
 inline hipStream_t st(void *s) { return static_cast<hipStream_t>(s); }
 
 // The weight-streaming kernel wins while a row tile of twice the mean rows per expert is
-// at most 64 rows (measured crossover against the 128x128 MFMA tiles on MI355X).
+// at most 64 rows (measured crossover against the 128x256 MFMA tiles on MI355X).
 constexpr int64_t kStreamMaxRowsPerExpert = 64;
 
 int env_int(const char *name, int dflt)
@@ -82,13 +82,13 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
         return launch_gemm_stream(X, off, W, B, E, R, K, N, dtype, epilogue, hint,
                                   env_int("OPMX_MOE_GEMM_STREAM_VARIANT", 0), Y, s);
     if (choice == 2) {
-        // Direct-to-LDS kernel from 128 mean rows per expert on, else 128x128 register-staged
-        // (measured).  The direct-to-LDS kernel takes 256x256 tiles unless they would fill the CUs
-        // less than twice (the Mixtral down projection at T=2048: 1.3 rounds): then 128x256 tiles,
-        // 20 % slower per flop but with half the quantisation (-9 % there).
+        // The direct-to-LDS kernel takes 256x256 tiles unless they would fill the CUs less than
+        // twice (the Mixtral down projection at T=2048: 1.3 rounds) or the experts hold fewer than
+        // 128 rows on average: then 128x256 tiles, 20 % slower per flop but with half the
+        // quantisation (-9 % at T=2048; at T=256 8 % faster than 128x128 register-staged tiles).
         const int64_t out_cols = epilogue == OPMX_EPILOGUE_SWIGLU ? N / 2 : N;
         const int64_t tiles256 = (R / 256 + (E + 1) / 2) * ((out_cols + 255) / 256);
-        const int dflt = R / E >= 128 ? (tiles256 < 512 ? 3 : 0) : 2;
+        const int dflt = R / E >= 128 && tiles256 >= 512 ? 0 : 3;
         return launch_gemm_tiled(X, off, W, B, E, R, K, N, dtype, epilogue,
                                  env_int("OPMX_MOE_GEMM_TILED_VARIANT", dflt), Y, ws, ws_bytes, s);
     }

@@ -4,7 +4,8 @@
 // the flops ride along on v_mfma_f32_16x16x32 with W as the A operand (16 weight
 // rows per wave) and the expert's few X rows as the B operand.
 //
-//  * a block = 4 waves = 64 consecutive rows of W[e] (one 16-row group per wave)
+//  * a block = 4 waves = 64 consecutive rows of W[e] (one 16-row group per wave; two groups,
+//    128 rows per block, once the row tile is 64 rows or taller)
 //    x one row tile (<= 16*MT rows) of expert e, over the whole K;
 //  * W is fetched with fully coalesced 16-byte loads (a wave instruction reads
 //    1 KiB contiguous) into registers, DEPTH K-chunks ahead, then transposed
@@ -31,15 +32,20 @@ template <bool NT> __device__ __forceinline__ u32x4 ld16(const char *p)
     return *reinterpret_cast<const u32x4 *>(p);
 }
 
-template <typename T, int MT, int KC, int DEPTH, bool NT, int SW, bool SG>
+template <typename T, int MT, int KC, int DEPTH, bool NT, int SW, bool SG, bool PAIR>
 __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restrict__ X,
                                                                const int64_t *__restrict__ off,
                                                                const T *__restrict__ W,
                                                                const T *__restrict__ Bias, int E, int64_t R,
                                                                int64_t K, int64_t N, T *__restrict__ Y)
 {
-    constexpr int NG = SG ? 2 : 1;               // row groups per wave: SwiGLU pairs gate rows with up rows
-    constexpr int SROWS = 16 * SW;               // output columns per block
+    // row groups per wave: SwiGLU pairs gate rows with up rows; PAIR gives a wave two adjacent
+    // groups, so that a block shares its X chunk among twice the weight rows (tall row tiles,
+    // where the X chunk is as large as the weight chunk)
+    static_assert(!(SG && PAIR), "one or the other");
+    constexpr int NG = (SG || PAIR) ? 2 : 1;
+    constexpr int WROWS = PAIR ? 32 : 16;        // output columns per wave
+    constexpr int SROWS = WROWS * SW;            // output columns per block
     constexpr int RS = KC * 2 + 16;              // LDS row stride in bytes (pad 16: conflict-free strips)
     constexpr int RPL = 512 / KC;                // W rows covered by one wave load (1 KiB)
     constexpr int NLW = 16 / RPL;                // W loads per wave per chunk
@@ -66,7 +72,7 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
 
     // ---- this wave's 16 rows of W[e]: uniform base + per-lane byte offsets.
     // Rows past N are clamped to row N-1 (their results are masked at the store).
-    const int64_t nbase = static_cast<int64_t>(blockIdx.x) * SROWS + wave * 16;
+    const int64_t nbase = static_cast<int64_t>(blockIdx.x) * SROWS + wave * WROWS;
     const char *wb = reinterpret_cast<const char *>(W + static_cast<int64_t>(mt.e) * N * K);
     const char *xb = reinterpret_cast<const char *>(X + mt.row0 * K);
     const int wl_row = lane / (64 / RPL);               // row inside one wave load
@@ -78,8 +84,8 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
 #pragma unroll
         for (int i = 0; i < NLW; ++i) {
             const int row = i * RPL + wl_row;
-            int64_t n = nbase + row;
-            n = (n < ND ? n : ND - 1) + g * ND;
+            int64_t n = nbase + row + (PAIR ? g * 16 : 0);
+            n = (n < ND ? n : ND - 1) + (SG ? g * ND : 0);
             wrow[g][i] = static_cast<uint32_t>(n * K * 2);
             wdst[g][i] = (g * 16 + row) * RS + wl_k * 2;
         }
@@ -187,29 +193,31 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
         if (row >= mt.rows) continue;
         T *yrow = Y + (mt.row0 + row) * ND;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int64_t n = nbase + fg * 4 + i;
-            if (n >= ND) continue;
-            float v = acc[0][m][i];
-            if (Bias) v += to_f32(Bias[static_cast<int64_t>(mt.e) * N + n]);
-            if (SG) {                          // SwiGLU.py:15-16 on the fp32 accumulators, beta = 1
-                float u = acc[NG - 1][m][i];
-                if (Bias) u += to_f32(Bias[static_cast<int64_t>(mt.e) * N + ND + n]);
-                v = u * v * sigmoid_fast_(v);
+        for (int g = 0; g < (PAIR ? 2 : 1); ++g)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int64_t n = nbase + g * 16 + fg * 4 + i;
+                if (n >= ND) continue;
+                float v = acc[g][m][i];
+                if (Bias) v += to_f32(Bias[static_cast<int64_t>(mt.e) * N + n]);
+                if (SG) {                          // SwiGLU.py:15-16 on the fp32 accumulators, beta = 1
+                    float u = acc[NG - 1][m][i];
+                    if (Bias) u += to_f32(Bias[static_cast<int64_t>(mt.e) * N + ND + n]);
+                    v = u * v * sigmoid_fast_(v);
+                }
+                yrow[n] = from_f32<T>(v);
             }
-            yrow[n] = from_f32<T>(v);
-        }
     }
 }
 
-template <typename T, int MT, int KC, int DEPTH, bool NT, int SW, bool SG>
+template <typename T, int MT, int KC, int DEPTH, bool NT, int SW, bool SG, bool PAIR = false>
 int stream_launch_sw(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
                      int64_t N, void *Y, hipStream_t s)
 {
-    constexpr int SROWS = 16 * SW;
+    constexpr int SROWS = (PAIR ? 32 : 16) * SW;
     constexpr int RS = KC * 2 + 16;
-    constexpr int smem = SW * (SG ? 2 : 1) * 16 * RS + 2 * 16 * MT * RS;
-    auto kern = gemm_stream_kernel<T, MT, KC, DEPTH, NT, SW, SG>;
+    constexpr int smem = SW * ((SG || PAIR) ? 2 : 1) * 16 * RS + 2 * 16 * MT * RS;
+    auto kern = gemm_stream_kernel<T, MT, KC, DEPTH, NT, SW, SG, PAIR>;
     static bool attr_done = false;
     if (!attr_done) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -232,6 +240,11 @@ int stream_launch(const void *X, const int64_t *off, const void *W, const void *
     const int64_t items = ceil_div(SG ? N / 2 : N, 64) * (R < E ? R : E);
     if (MT <= 2 && items < 512)
         return stream_launch_sw<T, MT, KC, DEPTH, NT, 1, SG>(X, off, W, B, E, R, K, N, Y, s);
+    // Tall row tiles: the X chunk a block stages is as large as its weight chunk, so every wave takes
+    // two groups of weight rows and the block shares X among 128 of them (Mixtral gate/up at
+    // T = 128: 357 -> 337 us, 64-row tiles; T = 256, 128-row tiles: 497 -> 374 us).
+    if constexpr (MT >= 4 && !SG)
+        return stream_launch_sw<T, MT, KC, DEPTH, NT, 4, SG, true>(X, off, W, B, E, R, K, N, Y, s);
     return stream_launch_sw<T, MT, KC, DEPTH, NT, 4, SG>(X, off, W, B, E, R, K, N, Y, s);
 }
 
