@@ -45,7 +45,7 @@ size_t grouped_gemm_workspace_bytes(int E, int64_t R, int64_t K, int64_t N, int 
 {
     (void)N;
     const bool lowp = dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16;
-    if (lowp && E > 0 && K > 0 && K % 64 == 0 && R / E >= 128) {
+    if (lowp && E > 0 && K > 0 && K % 64 == 0 && 2 * ceil_div(R, E) > kStreamMaxRowsPerExpert) {
         const size_t b = gemm_tiled_workspace_bytes();
         if (b > 0) return (b + 255) / 256 * 256;
     }
