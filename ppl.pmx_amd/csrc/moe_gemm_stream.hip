@@ -256,9 +256,21 @@ template <typename T, int KC1, int KC2, int KC4, int KC8, int DEPTH, bool NT>
 int stream_pick_mt(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
                    int64_t N, int64_t m, void *Y, hipStream_t s)
 {
-    if (m <= 2) return stream_launch<T, 1, KC1, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
-    if (m <= 32) return stream_launch<T, 2, KC2, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
-    if (m <= 64) return stream_launch<T, 4, KC4, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
+    // A short K (fewer than 16 chunks of 256) is walked in chunks of 128: a block then lives for a
+    // few chunks only, and the narrower chunks halve its LDS footprint, so that twice as many
+    // blocks per CU overlap each other's start and end (64 experts, H = 2048, I = 1408, bf16:
+    // layer at T = 32 0.255 -> 0.211 ms, at T = 1 0.189 -> 0.126 ms).
+    constexpr int KC1S = KC1 > 128 ? 128 : KC1, KC2S = KC2 > 128 ? 128 : KC2, KC4S = KC4 > 64 ? 64 : KC4;
+    const bool short_k = K < 16 * 256;
+    if (m <= 2)
+        return short_k ? stream_launch<T, 1, KC1S, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s)
+                       : stream_launch<T, 1, KC1, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
+    if (m <= 32)
+        return short_k ? stream_launch<T, 2, KC2S, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s)
+                       : stream_launch<T, 2, KC2, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
+    if (m <= 64)
+        return short_k ? stream_launch<T, 4, KC4S, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s)
+                       : stream_launch<T, 4, KC4, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
     return stream_launch<T, 8, KC8, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
 }
 
@@ -268,7 +280,9 @@ int stream_swiglu_impl(const void *X, const int64_t *off, const void *W, const v
                        int64_t N, int64_t rows_hint, void *Y, hipStream_t s)
 {
     const int64_t m = rows_hint > 0 ? rows_hint : R;
-    if (m <= 2) return stream_launch<T, 1, 256, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);
+    if (m <= 2)      // short K: narrower chunks, as in stream_pick_mt
+        return K < 16 * 256 ? stream_launch<T, 1, 128, 2, true, true>(X, off, W, B, E, R, K, N, Y, s)
+                            : stream_launch<T, 1, 256, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);
     if (m <= 32) return stream_launch<T, 2, 128, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);
     if (m <= 64) return stream_launch<T, 4, 64, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);
     return stream_launch<T, 8, 64, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);

@@ -188,6 +188,12 @@ def test_stream_kernel_variants(variant, dtype):
     # also through a ragged last chunk and in the SwiGLU form
     run_case("row", [8, 9, 7, 11, 0, 16, 5, 8], 8192 + 72, 320, dtype, True, env)
     run_case("column", [30, 2, 17, 0, 32, 1, 25, 21], 4096, 2 * 192, dtype, False, env, swiglu=True)
+    # K below 4096 takes narrower K chunks (all the cases above but the last two): the wide-chunk
+    # kernels for single rows and for 64-row tiles, and the narrow SwiGLU one for single rows
+    run_case("column", [1, 0, 1, 0, 0, 0, 0, 0], 4096, 192, dtype, True, env)
+    run_case("row", [64, 40, 0, 3, 50, 33, 1, 65], 4096 + 64, 192, dtype, False, env)
+    run_case("column", [1, 0, 1, 0, 0, 0, 1, 0], 1408, 2 * 128, dtype, True, env, swiglu=True)
+    run_case("column", [1, 0, 1, 0, 0, 0, 1, 0], 4096, 2 * 128, dtype, False, env, swiglu=True)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
