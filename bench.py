@@ -11,6 +11,8 @@ already resident in HBM.  Prints ONE JSON line:
                        or flops per launch / mean launch duration (HIP events on
                        the launch stream, taken inside the timed steps) vs MI355X peak
   layer                the same accounting for the whole layer
+  hip_graph_replay     the same steps replayed from one captured HIP graph (launch cost of the
+                       six operators taken off the host)
   per_op_us            mean duration of each operator (separate untimed pass)
   device_ceilings      streaming-read GB/s and MFMA TFLOP/s (random fp16 operands) this
                        device sustains, from the probe ppl.pmx_amd/lib/opmx_device_ceilings
@@ -69,6 +71,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="decode-T32")
+    ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay leg")
     ap.add_argument("--fuse-swiglu", action="store_true", help="apply SwiGLU in the gate/up GEMM epilogue")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg")
@@ -115,7 +118,7 @@ def main():
                 line = subprocess.run(cmd, capture_output=True, text=True, timeout=300, check=True).stdout.strip().splitlines()[-1]
                 r = json.loads(line)
                 companion[name] = {key: r[key] for key in ("value", "unit", "ms_per_step", "steps", "config", "roofline",
-                                                           "layer", "per_op_us")}
+                                                           "layer", "hip_graph_replay", "per_op_us")}
             except Exception as exc:
                 print("companion workload failed: {}".format(exc), file=sys.stderr)
 
@@ -196,6 +199,28 @@ def main():
         dt = time.perf_counter() - t0
         ms_per_step = dt / args.steps * 1e3
         gemm1_ms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
+
+        # ---- the same steps replayed from a captured HIP graph: what a serving loop does when the
+        # host's launch path (six operators per layer) is slower than the GPU work, i.e. at few
+        # tokens.  Reported beside `value`, which stays the eager operator sequence.
+        graph_ms = None
+        if not args.no_graph:
+            try:
+                torch.cuda.synchronize()
+                cg = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(cg):
+                    ops()
+                for _ in range(max(args.warmup, 1)):
+                    cg.replay()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(args.steps):
+                    cg.replay()
+                torch.cuda.synchronize()
+                graph_ms = (time.perf_counter() - t0) / args.steps * 1e3
+                del cg
+            except Exception as exc:
+                print("graph replay leg failed: {}".format(exc), file=sys.stderr)
 
         # ---- per-operator durations (untimed extra pass, averaged)
         per_op = {}
@@ -278,7 +303,10 @@ def main():
             cfg["name"], "decode" if hbm_bound else "prefill", T, H, E, k, I),
             "path": "drop-in operator sequence" + (" + fused SwiGLU epilogue" if args.fuse_swiglu else ""),
             "active_experts": active, "max_expert_share": round(float(counts.max()) / R, 3)},
-        "roofline": roof, "layer": lay, "per_op_us": {n: round(v, 1) for n, v in per_op.items()},
+        "roofline": roof, "layer": lay,
+        "hip_graph_replay": None if graph_ms is None else {"ms_per_step": round(graph_ms, 4),
+                                                           "value": round(T / (graph_ms * 1e-3), 1), "unit": "tokens/s"},
+        "per_op_us": {n: round(v, 1) for n, v in per_op.items()},
         "device_ceilings": ceilings, "companion": companion, "vendor_dense_gemm_same_flops_TFLOPs": vendor_tflops, "device": torch.cuda.get_device_name(0), "cu_count": torch.cuda.get_device_properties(0).multi_processor_count,
     }
 
