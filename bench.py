@@ -45,8 +45,8 @@ MFMA_PEAK_TFLOPS = 2500.0      # dense fp16/bf16 MFMA, vendor figure
 # (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000): profiles/gemm_stream_decode_T32_mixtral8x7b.txt and
 # profiles/gemm_tiled_prefill_T8192_mixtral8x7b.txt.  None where no counter run was made.
 MEASURED_TRAFFIC = {
-    ("decode-T32", False): 1883389952 + 3674726,
-    ("prefill-T8192", False): 2 * 4160709 * 1024 + 917504 * 1024,
+    ("decode-T32", False): 1883394048 + 3674624,
+    ("prefill-T8192", False): 2 * 3859194 * 1024 + 917504 * 1024,
 }
 
 SHAPES = {
