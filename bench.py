@@ -72,6 +72,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="decode-T32")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay leg")
+    ap.add_argument("--fuse-router-select", action="store_true",
+                    help="router gate and MoeSelect through the fused call (one launch up to 8 tokens)")
     ap.add_argument("--fuse-swiglu", action="store_true", help="apply SwiGLU in the gate/up GEMM epilogue")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg")
@@ -158,8 +160,11 @@ def main():
             b.record()
             record.append((name, a, b))
             return r
-        sc = timed("router_linear", lambda: OPMX.linear(x, Wg, gb, H, E))
-        xe, w, inv, off = timed("moe_select", lambda: OPMX.moe_select(x, sc, E, k))
+        if args.fuse_router_select:
+            xe, w, inv, off, sc = timed("router_and_select", lambda: OPMX.moe_route_select(x, Wg, gb, E, k))
+        else:
+            sc = timed("router_linear", lambda: OPMX.linear(x, Wg, gb, H, E))
+            xe, w, inv, off = timed("moe_select", lambda: OPMX.moe_select(x, sc, E, k))
         if args.fuse_swiglu:
             act = timed("gate_up_gemm", lambda: OPMX.moe_column_parallel_linear_swiglu(xe, off, wu, None, E, H, 2 * I))
         else:
@@ -187,8 +192,11 @@ def main():
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for i in range(args.steps):
-            sc = OPMX.linear(x, Wg, gb, H, E)
-            xe, w, inv, off = OPMX.moe_select(x, sc, E, k)
+            if args.fuse_router_select:
+                xe, w, inv, off, sc = OPMX.moe_route_select(x, Wg, gb, E, k)
+            else:
+                sc = OPMX.linear(x, Wg, gb, H, E)
+                xe, w, inv, off = OPMX.moe_select(x, sc, E, k)
             ev[i][0].record()
             h = gemm1(xe, off)
             ev[i][1].record()
@@ -301,7 +309,8 @@ def main():
         "dtype": {"float16": "f16", "bfloat16": "bf16"}[cfg["dtype"]], "data": "synthetic",
         "config": {"workload": "{} MoE layer {}, T={} tokens, hidden={}, experts={}, top-{}, ffn={}, TP=1".format(
             cfg["name"], "decode" if hbm_bound else "prefill", T, H, E, k, I),
-            "path": "drop-in operator sequence" + (" + fused SwiGLU epilogue" if args.fuse_swiglu else ""),
+            "path": "drop-in operator sequence" + (" + fused SwiGLU epilogue" if args.fuse_swiglu else "")
+            + (" + router gate and select in one call" if args.fuse_router_select else ""),
             "active_experts": active, "max_expert_share": round(float(counts.max()) / R, 3)},
         "roofline": roof, "layer": lay,
         "hip_graph_replay": None if graph_ms is None else {"ms_per_step": round(graph_ms, 4),

@@ -88,6 +88,23 @@ int opmx_moe_select(const void *X, const void *scores, int64_t T, int64_t H, int
                     int64_t *invert_permutation, int64_t *expert_offset, int32_t *expert_ids,
                     void *workspace, size_t workspace_bytes, void *stream);
 
+/* Router gate and MoeSelect in one call: scores = X gate_weight^T (+ gate_bias), then
+ * opmx_moe_select on those scores.  Replaces the pair of calls at
+ * model_zoo/mixtral/modeling/dynamic_batching/Model.py:188-190 (self.gate, then
+ * OPMX.moe_select); the two operators stay callable on their own.
+ *   X [T,H], gate_weight [E,H], gate_bias [E] or NULL          (dtype)
+ *   scores [T,E]: receives the router logits (an input of opmx_moe_select, an output here)
+ *   the other outputs, the limits and the workspace are those of opmx_moe_select.
+ * fp16/bf16 with T <= 8, E <= 16, H % 32 == 0 and 16-byte aligned X / gate_weight run as a
+ * single launch (every block recomputes the few logits on the MFMA units); anything else runs
+ * opmx_linear and opmx_moe_select one after the other.  Routing is exact on the returned
+ * scores; the scores themselves may differ from opmx_linear's in the last bit (other
+ * summation order of the fp32 accumulation). */
+int opmx_moe_route_select(const void *X, const void *gate_weight, const void *gate_bias, int64_t T,
+                          int64_t H, int E, int k, int dtype, void *scores, void *X_expand_permute,
+                          void *expert_weights, int64_t *invert_permutation, int64_t *expert_offset,
+                          int32_t *expert_ids, void *workspace, size_t workspace_bytes, void *stream);
+
 /* Grouped expert GEMM.  Replaces the per-expert F.linear loops of
  * MoeColumnParallelLinear.forward (torch_function/MoeColumnParallelLinear.py:58-69)
  * and MoeRowParallelLinear.forward (torch_function/MoeRowParallelLinear.py:44-60)

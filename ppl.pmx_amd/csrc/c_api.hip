@@ -144,6 +144,24 @@ int opmx_moe_select(const void *X, const void *scores, int64_t T, int64_t H, int
                              expert_offset, expert_ids, workspace, st(stream));
 }
 
+int opmx_moe_route_select(const void *X, const void *gate_weight, const void *gate_bias, int64_t T, int64_t H, int E,
+                          int k, int dtype, void *scores, void *X_expand_permute, void *expert_weights,
+                          int64_t *invert_permutation, int64_t *expert_offset, int32_t *expert_ids, void *workspace,
+                          size_t workspace_bytes, void *stream)
+{
+    if (T < 0 || H < 0 || E <= 0 || k <= 0 || k > E) return OPMX_ERR_BAD_ARGUMENT;
+    if (!dtype_ok(dtype) || E > OPMX_MOE_MAX_EXPERTS || k > OPMX_MOE_MAX_EXPERTS_PER_TOKEN)
+        return OPMX_ERR_UNSUPPORTED;
+    if (T > (int64_t{1} << 31) / k) return OPMX_ERR_UNSUPPORTED;
+    if (!expert_offset) return OPMX_ERR_BAD_ARGUMENT;
+    if (T > 0 && (!scores || !expert_weights || !invert_permutation)) return OPMX_ERR_BAD_ARGUMENT;
+    if (T > 0 && H > 0 && (!X || !gate_weight || !X_expand_permute)) return OPMX_ERR_BAD_ARGUMENT;
+    if (T > 0 && (!workspace || workspace_bytes < moe_select_workspace_bytes(T, E, k))) return OPMX_ERR_WORKSPACE;
+    if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 255u)) return OPMX_ERR_ALIGNMENT;
+    return launch_moe_route_select(X, gate_weight, gate_bias, T, H, E, k, dtype, scores, X_expand_permute,
+                                   expert_weights, invert_permutation, expert_offset, expert_ids, workspace, st(stream));
+}
+
 size_t opmx_moe_grouped_gemm_workspace_bytes(int E, int64_t R, int64_t K, int64_t N, int dtype)
 {
     return grouped_gemm_workspace_bytes(E, R, K, N, dtype);

@@ -80,6 +80,9 @@ int launch_moe_select(const void *X, const void *scores, int64_t T, int64_t H, i
                       void *Xp, void *w, int64_t *inv, int64_t *off, int32_t *ids, void *ws,
                       hipStream_t s);
 size_t moe_select_workspace_bytes(int64_t T, int E, int k);
+int launch_moe_route_select(const void *X, const void *Wg, const void *Bg, int64_t T, int64_t H, int E, int k,
+                            int dtype, void *scores, void *Xp, void *w, int64_t *inv, int64_t *off, int32_t *ids,
+                            void *ws, hipStream_t s);
 int launch_swiglu(const void *X, int64_t R, int64_t D, float beta, int dtype, void *Y, hipStream_t s);
 int launch_silu(const void *X, const void *gate, int64_t n, int dtype, void *Y, hipStream_t s);
 int launch_rms_norm(const void *X, const void *Wt, const void *Skip, int64_t T, int64_t H, float eps, int dtype,

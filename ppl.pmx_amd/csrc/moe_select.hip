@@ -6,7 +6,7 @@
 //   expert_offset[e] + (#tokens before it that picked e)
 // and the count is taken from bit matrices (one bit per (expert, token)), whose
 // construction by atomicOr is order independent.
-#include "common.h"
+#include "moe_gemm.h"
 
 namespace opmx {
 namespace {
@@ -282,24 +282,93 @@ __global__ __launch_bounds__(256) void select_expand_kernel(const T *__restrict_
     for (int64_t t = blockIdx.x; t < Ttok; t += gridDim.x) expand_row(X, Xp, t, H, k, inv + t * k, vec);
 }
 
+// Router logits of up to kFusedTokens tokens and kFusedExperts experts, computed by one
+// 1024-thread block into LDS: scores[t][e] = X[t] . Wg[e] (+ Bg[e]), fp32 accumulation on the MFMA
+// 16x16x32 units, rounded once to T (Linear.py:32).  The sixteen waves split K (a wave's few
+// k-steps are in flight together: the phase costs about one memory round trip); their partial
+// sums meet in LDS and are added in wave order, so the result does not depend on timing.  Every
+// block of the fused kernel computes all logits redundantly, which is what lets one launch do
+// router gate and routing without a grid-wide exchange -- and what limits it to few tokens.
+// Measured on the Mixtral shape: one launch saves 1 us per layer at T = 1, breaks even at T = 8,
+// costs 1-2 us at T = 16 (3-4 us with H = 6144) and 4.5 us at T = 32 (a two-tile form): a
+// dependent launch on the same stream is cheap here, recomputing the logits per block is not.
+// So one launch serves up to kFusedMaxTokens tokens; more go to the two separate kernels.
+constexpr int kFusedTokens = 16, kFusedExperts = 16, kFusedWaves = 16;   // what the kernel can do
+constexpr int kFusedMaxTokens = 8;                                       // what it is used for
+template <typename T>
+__device__ __forceinline__ void router_logits_to_lds(const T *__restrict__ X, const T *__restrict__ Wg,
+                                                     const T *__restrict__ Bg, int Ttok, int64_t H, int E,
+                                                     float *part /* [kFusedWaves][64][4] */, T *s_scores /* [Ttok*E] */)
+{
+    using frag = typename Mfma<T>::frag;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int fr = lane & 15, fg = lane >> 4;
+    const int erow = fr < E ? fr : E - 1;               // padded expert rows repeat the last one
+    const int trow = fr < Ttok ? fr : Ttok - 1;         // padded token rows likewise
+    const T *wp = Wg + static_cast<int64_t>(erow) * H + fg * 8;
+    const T *xp = X + static_cast<int64_t>(trow) * H + fg * 8;
+    float4_t acc = {0.f, 0.f, 0.f, 0.f};
+    const int steps = static_cast<int>(H / 32);
+    int st = wave;                      // wave w takes k-steps w, w+16, ... in this order
+    for (; st + 3 * kFusedWaves < steps; st += 4 * kFusedWaves) {   // four steps' loads in flight
+        frag a[4], b[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            a[u] = *reinterpret_cast<const frag *>(wp + (st + kFusedWaves * u) * 32);
+            b[u] = *reinterpret_cast<const frag *>(xp + (st + kFusedWaves * u) * 32);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) acc = Mfma<T>::m16(a[u], b[u], acc);
+    }
+    for (; st < steps; st += kFusedWaves) {
+        const frag a = *reinterpret_cast<const frag *>(wp + st * 32);
+        const frag b = *reinterpret_cast<const frag *>(xp + st * 32);
+        acc = Mfma<T>::m16(a, b, acc);
+    }
+    // acc[i]: expert fg*4 + i, token fr
+    *reinterpret_cast<float4_t *>(part + (wave * 64 + lane) * 4) = acc;
+    __syncthreads();
+    for (int q = threadIdx.x; q < Ttok * E; q += blockDim.x) {
+        const int t = q / E, e = q % E;
+        const int idx = ((e >> 2) * 16 + t) * 4 + (e & 3);
+        float v = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kFusedWaves; ++w) v += part[w * 64 * 4 + idx];
+        if (Bg) v += to_f32(Bg[e]);
+        s_scores[q] = from_f32<T>(v);
+    }
+    __syncthreads();
+}
+
 // ---- small-T path: one launch.  Every block routes all T <= kChunk tokens
 // redundantly in LDS, then block b emits the outputs of token b and copies its row.
-template <typename T>
+// FUSED: the router logits are computed here as well (scores = X Wg^T + Bg, T <= kFusedTokens,
+// E <= kFusedExperts, 1024 threads) and written to `scores_out`, each block its own token's row.
+template <typename T, bool FUSED>
 __global__ __launch_bounds__(1024) void select_small_kernel(const T *__restrict__ X,
                                                               const T *__restrict__ scores, int Ttok,
                                                               int64_t H, int E, int k, int G, int vpl,
                                                               T *__restrict__ Xp, T *__restrict__ weights,
                                                               int64_t *__restrict__ inv,
                                                               int64_t *__restrict__ off,
-                                                              int32_t *__restrict__ ids_out, bool vec)
+                                                              int32_t *__restrict__ ids_out, bool vec,
+                                                              const T *__restrict__ Wg, const T *__restrict__ Bg,
+                                                              T *__restrict__ scores_out)
 {
     __shared__ uint32_t bits[OPMX_MOE_MAX_EXPERTS * kWords];
     __shared__ int wordpre[OPMX_MOE_MAX_EXPERTS * kWords];
     __shared__ int count[OPMX_MOE_MAX_EXPERTS + 1];
     __shared__ int my_ids[OPMX_MOE_MAX_EXPERTS_PER_TOKEN];
     __shared__ int64_t my_inv[OPMX_MOE_MAX_EXPERTS_PER_TOKEN];
+    __shared__ __attribute__((aligned(16))) float part[FUSED ? kFusedWaves * 64 * 4 : 4];
+    __shared__ T s_scores[FUSED ? kFusedTokens * kFusedExperts : 1];
     const int lig = threadIdx.x % G, grp = threadIdx.x / G, ngrp = blockDim.x / G;
     const int me = blockIdx.x;                 // the token this block emits
+    if constexpr (FUSED) {
+        if constexpr (sizeof(T) == 2) router_logits_to_lds<T>(X, Wg, Bg, Ttok, H, E, part, s_scores);
+        for (int e = threadIdx.x; e < E; e += blockDim.x) scores_out[static_cast<int64_t>(me) * E + e] = s_scores[me * E + e];
+        scores = s_scores;
+    }
     zero_bits(bits, E);
     __syncthreads();
     for (int tl = grp; tl < Ttok; tl += ngrp) {   // whole lane groups iterate together
@@ -364,8 +433,8 @@ int select_impl(const void *X_, const void *scores_, int64_t Ttok, int64_t H, in
     if (Ttok <= kChunk && Ttok * G <= kChunk * 8) {
         // wide lane groups (many experts) route few tokens per wave: use a big block
         const unsigned threads = G >= 32 ? 1024 : kChunk;
-        select_small_kernel<T><<<static_cast<unsigned>(Ttok), threads, 0, s>>>(
-            X, scores, static_cast<int>(Ttok), H, E, k, G, vpl, Xp, w, inv, off, ids, vec);
+        select_small_kernel<T, false><<<static_cast<unsigned>(Ttok), threads, 0, s>>>(
+            X, scores, static_cast<int>(Ttok), H, E, k, G, vpl, Xp, w, inv, off, ids, vec, nullptr, nullptr, nullptr);
         OPMX_LAUNCH_CHECK();
         return OPMX_OK;
     }
@@ -388,7 +457,43 @@ int select_impl(const void *X_, const void *scores_, int64_t Ttok, int64_t H, in
     return OPMX_OK;
 }
 
+template <typename T>
+int route_select_fused(const void *X_, const void *Wg_, const void *Bg_, int64_t Ttok, int64_t H, int E, int k,
+                       void *scores_, void *Xp_, void *w_, int64_t *inv, int64_t *off, int32_t *ids, hipStream_t s)
+{
+    const T *X = static_cast<const T *>(X_);
+    T *Xp = static_cast<T *>(Xp_);
+    int G = 8;
+    while (G < E) G <<= 1;
+    const bool vec = (H * sizeof(T)) % 16 == 0 && aligned16(X) && aligned16(Xp);
+    select_small_kernel<T, true><<<static_cast<unsigned>(Ttok), kFusedWaves * kWave, 0, s>>>(
+        X, nullptr, static_cast<int>(Ttok), H, E, k, G, (E + G - 1) / G, Xp, static_cast<T *>(w_), inv, off, ids, vec,
+        static_cast<const T *>(Wg_), static_cast<const T *>(Bg_), static_cast<T *>(scores_));
+    OPMX_LAUNCH_CHECK();
+    return OPMX_OK;
+}
+
 }  // namespace
+
+// Router gate and MoeSelect in one call.  One launch when the logits of all tokens fit one
+// MFMA tile per block and that pays (fp16/bf16, T <= 8, E <= 16, H a multiple of 32, 16-byte aligned rows);
+// otherwise the two operators one after the other.  `scores` [T,E] receives the logits either way.
+int launch_moe_route_select(const void *X, const void *Wg, const void *Bg, int64_t T, int64_t H, int E, int k,
+                            int dtype, void *scores, void *Xp, void *w, int64_t *inv, int64_t *off, int32_t *ids,
+                            void *ws, hipStream_t s)
+{
+    const bool lowp = dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16;
+    static_assert(kFusedMaxTokens <= kFusedTokens, "one MFMA tile of tokens");
+    if (lowp && T >= 1 && T <= kFusedMaxTokens && E <= kFusedExperts && H >= 32 && H % 32 == 0 && aligned16(X) &&
+        aligned16(Wg)) {
+        if (dtype == OPMX_DTYPE_F16)
+            return route_select_fused<f16>(X, Wg, Bg, T, H, E, k, scores, Xp, w, inv, off, ids, s);
+        return route_select_fused<bf16>(X, Wg, Bg, T, H, E, k, scores, Xp, w, inv, off, ids, s);
+    }
+    const int rc = launch_linear(X, Wg, Bg, T, H, E, dtype, scores, s);
+    if (rc != OPMX_OK) return rc;
+    return launch_moe_select(X, scores, T, H, E, k, dtype, Xp, w, inv, off, ids, ws, s);
+}
 
 size_t moe_select_workspace_bytes(int64_t T, int E, int k)
 {

@@ -30,15 +30,18 @@ class MoeFeedForward(nn.Module):
     ``fuse_swiglu_epilogue=True`` (only with ``fused_ffn_glu``) applies SwiGLU
     inside the gate/up GEMM instead of as a separate operator; results agree
     to rounding, the ONNX graph does not change because export always takes
-    the operator-by-operator route.
+    the operator-by-operator route.  ``fuse_router_select=True`` does the same for the router
+    gate and MoeSelect (one launch up to 8 tokens; the routing is exact on the logits that
+    launch computes, which can differ from the separate gate's in the last bit).
     """
 
     def __init__(self, args, layer_id: int, fused_ffn_glu: bool, linear_bias_term: bool, proc_group,
-                 dtype=None, device=None, fuse_swiglu_epilogue: bool = False):
+                 dtype=None, device=None, fuse_swiglu_epilogue: bool = False, fuse_router_select: bool = False):
         super().__init__()
         self.layer_id = layer_id
         self.fused_ffn_glu = fused_ffn_glu
         self.fuse_swiglu_epilogue = fuse_swiglu_epilogue and fused_ffn_glu
+        self.fuse_router_select = fuse_router_select
         self.num_experts = args.num_experts
         self.num_experts_per_token = args.num_experts_per_token
         kw = dict(dtype=dtype, device=device)
@@ -62,9 +65,13 @@ class MoeFeedForward(nn.Module):
 
     def forward(self, x):
         k = self.num_experts_per_token
-        router_logits = self.gate(x)
-        x_experts, expert_weights, invert_permutation, expert_offset = OPMX.moe_select(
-            x, router_logits, self.num_experts, k)
+        if self.fuse_router_select and not torch.onnx.is_in_onnx_export():
+            x_experts, expert_weights, invert_permutation, expert_offset, _ = OPMX.moe_route_select(
+                x, self.gate.weight, self.gate.bias, self.num_experts, k)
+        else:
+            router_logits = self.gate(x)
+            x_experts, expert_weights, invert_permutation, expert_offset = OPMX.moe_select(
+                x, router_logits, self.num_experts, k)
         if self.fused_ffn_glu:
             if self.fuse_swiglu_epilogue and not torch.onnx.is_in_onnx_export():
                 x13 = OPMX.moe_column_parallel_linear_swiglu(
@@ -126,7 +133,7 @@ class MoeFeedForward(nn.Module):
 
 
 def load_opmx_moe_block(path, layer_id: int, num_experts_per_token: int, fused_ffn_glu: bool = True,
-                        dtype=None, device=None, fuse_swiglu_epilogue: bool = False):
+                        dtype=None, device=None, fuse_swiglu_epilogue: bool = False, fuse_router_select: bool = False):
     """Builds the MoE block of layer ``layer_id`` from an OPMX Mixtral ``.pth`` checkpoint.
 
     The file is opened with ``weights_only=True`` and memory-mapped, so only this layer's tensors are
@@ -141,6 +148,6 @@ def load_opmx_moe_block(path, layer_id: int, num_experts_per_token: int, fused_f
     bias = (prefix + "w2.bias") in sd
     block = MoeFeedForward(MoeFeedForward.params(H, w2.shape[2], E, num_experts_per_token), layer_id, fused_ffn_glu,
                            bias, None, dtype=gate.dtype if dtype is None else dtype, device=device,
-                           fuse_swiglu_epilogue=fuse_swiglu_epilogue)
+                           fuse_swiglu_epilogue=fuse_swiglu_epilogue, fuse_router_select=fuse_router_select)
     block.load_state_dict(sd)
     return block

@@ -56,3 +56,41 @@ def moe_select(X: torch.Tensor, scores: torch.Tensor, num_experts: int, num_expe
     """-> (X_expand_permute [*,k,H], expert_weights [*,k], invert_permutation [*,k] i64,
     expert_offset [E+1] i64)"""
     return MoeSelect.apply(X, scores, num_experts, num_experts_per_token)
+
+
+def moe_route_select(X: torch.Tensor, gate_weight: torch.Tensor, gate_bias, num_experts: int,
+                     num_experts_per_token: int):
+    """Router gate and ``moe_select`` in one call (``Model.py:188-190`` of the reference:
+    ``router_logits = self.gate(x)`` followed by ``OPMX.moe_select``).
+
+    -> the four outputs of ``moe_select`` plus the router logits ``[*, E]``.  Few tokens
+    (fp16/bf16, at most 8 tokens and 16 experts) run as a single launch; other sizes run the two
+    operators one after the other inside the library.  Not an ONNX node: a model that is being
+    exported calls ``linear`` and ``moe_select``.
+    """
+    E, k = int(num_experts), int(num_experts_per_token)
+    lead, H = tuple(X.shape[:-1]), X.shape[-1]
+    dev = _lib.require_gpu("moe_route_select", X, gate_weight, gate_bias)
+    if tuple(gate_weight.shape) != (E, H):
+        raise ValueError("moe_route_select: gate weight {} does not match [num_experts, hidden] = [{}, {}]".format(
+            tuple(gate_weight.shape), E, H))
+    if gate_weight.dtype != X.dtype or (gate_bias is not None and gate_bias.dtype != X.dtype):
+        raise TypeError("moe_route_select: X, gate weight and gate bias must share one dtype")
+    if not (1 <= k <= E):
+        raise ValueError("moe_route_select: need 1 <= num_experts_per_token <= num_experts")
+    dt = _lib.dtype_id(X, "moe_route_select")
+    Xf = X.reshape(-1, H).contiguous()
+    Wg = gate_weight.contiguous()
+    Bg = None if gate_bias is None else gate_bias.contiguous()
+    T = Xf.shape[0]
+    scores = torch.empty(T, E, dtype=X.dtype, device=dev)
+    x_expand = torch.empty(T * k, H, dtype=X.dtype, device=dev)
+    weights = torch.empty(T, k, dtype=X.dtype, device=dev)
+    inv = torch.empty(T * k, dtype=torch.int64, device=dev)
+    off = torch.empty(E + 1, dtype=torch.int64, device=dev)
+    L = _lib.lib()
+    ws = _lib.workspace(L.opmx_moe_select_workspace_bytes(T, E, k), dev)
+    _lib.check(L.opmx_moe_route_select(_lib.ptr(Xf), _lib.ptr(Wg), _lib.ptr(Bg), T, H, E, k, dt, _lib.ptr(scores),
+                                       _lib.ptr(x_expand), _lib.ptr(weights), _lib.ptr(inv), _lib.ptr(off), None,
+                                       _lib.ptr(ws), ws.numel(), _lib.stream_ptr(dev)), "moe_route_select")
+    return (x_expand.view(*lead, k, H), weights.view(*lead, k), inv.view(*lead, k), off, scores.view(*lead, E))

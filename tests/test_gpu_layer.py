@@ -14,22 +14,26 @@ pytestmark = pytest.mark.gpu
 MAX_ABS, MEAN_ABS = 2e-2, 2e-3
 
 
-def build_layer(H, I, E, k, dtype, Wg, wu, w2, fuse=False):
+def build_layer(H, I, E, k, dtype, Wg, wu, w2, fuse=False, route=False):
     from model_zoo.mixtral.modeling.dynamic_batching.Model import MoeFeedForward
     m = MoeFeedForward(MoeFeedForward.params(H, I, E, k), 0, True, False, None, dtype=dtype, device=dev(),
-                       fuse_swiglu_epilogue=fuse)
+                       fuse_swiglu_epilogue=fuse, fuse_router_select=route)
     m.gate.weight.data = Wg
     m.wu.weight.data = wu
     m.w2.weight.data = w2
     return m
 
 
-def run_ops(x, Wg, wu, w2, E, k, bias=None):
-    """The reference call sequence (Model.py:187-214) through the drop-in operators."""
+def run_ops(x, Wg, wu, w2, E, k, bias=None, route=False):
+    """The reference call sequence (Model.py:187-214) through the drop-in operators; `route`:
+    router gate and MoeSelect through the fused call."""
     import torch_function as OPMX
     H, I = x.shape[-1], w2.shape[-1]
-    scores = OPMX.linear(x, Wg, bias, H, E)
-    xe, w, inv, off = OPMX.moe_select(x, scores, E, k)
+    if route:
+        xe, w, inv, off, scores = OPMX.moe_route_select(x, Wg, bias, E, k)
+    else:
+        scores = OPMX.linear(x, Wg, bias, H, E)
+        xe, w, inv, off = OPMX.moe_select(x, scores, E, k)
     x13 = OPMX.moe_column_parallel_linear(xe, off, wu, None, None, E, H, 2 * I, False)
     act = OPMX.swiglu(x13)
     y = OPMX.moe_row_parallel_linear(act, off, w2, None, None, E, I, H, True)
@@ -95,6 +99,11 @@ def test_mixtral_8x7b_decode(mixtral_8x7b, T):
     mf = build_layer(4096, 14336, 8, 2, torch.float16, Wg, wu, w2, fuse=True)
     err = (mf(x[:T]).double() - g["out"].double()).abs()
     assert float(err.max()) <= MAX_ABS and float(err.mean()) <= MEAN_ABS
+    # router gate and select in one launch: the same bar on the logits that launch returns
+    gr = run_ops(x[:T], Wg, wu, w2, 8, 2, route=True)
+    check_against_oracle(gr, (host[0][:T],) + host[1:], 8, 2)
+    mr = build_layer(4096, 14336, 8, 2, torch.float16, Wg, wu, w2, route=True)
+    assert torch.equal(mr(x[:T]), gr["out"])
 
 
 @pytest.mark.parametrize("T,full", [(2048, True), (8192, False)])

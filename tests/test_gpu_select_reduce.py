@@ -185,3 +185,61 @@ def test_router_linear(T, K, N, dtype, bias):
     assert out.shape == (T, N) and out.dtype == dtype
     assert_close_ulp(out, ref, dtype, ulps=1.5 if dtype != torch.float32 else 32, what="linear",
                      floor=0.01 if dtype != torch.float32 else 0.25)
+
+
+# Router gate and MoeSelect in one call.  Up to 8 tokens and 16 experts in fp16/bf16 with
+# H % 32 == 0 it is a single launch whose logits come from the MFMA units; every other case runs
+# the two operators inside the library.  The bar is the same either way: the returned logits
+# within rounding of the fp32 oracle, and the routing bit-exact given those logits.
+ROUTE_SELECT_CASES = [
+    # T, H, E, k, dtype, bias
+    (1, 4096, 8, 2, torch.float16, False),      # Mixtral, one token
+    (8, 4096, 8, 2, torch.float16, True),       # largest single-launch size
+    (5, 1024, 16, 4, torch.bfloat16, True),     # 16 experts
+    (7, 96, 5, 2, torch.bfloat16, False),       # three k-steps for sixteen waves, E not a multiple of 4
+    (8, 32, 3, 3, torch.float16, True),         # one k-step: all waves but one add nothing
+    (8, 4096 + 32 * 67, 8, 2, torch.float16, True),    # k-steps not a multiple of the waves or of the unrolling
+    (9, 4096, 8, 2, torch.float16, True),       # one token too many: two launches
+    (32, 4096, 8, 2, torch.float16, True),      # Mixtral decode
+    (8, 2048, 64, 8, torch.bfloat16, False),    # too many experts
+    (8, 100, 8, 2, torch.float16, True),        # H not a multiple of 32
+    (8, 64, 8, 2, torch.float32, True),         # fp32
+    (600, 512, 16, 2, torch.float16, False),    # long prompt: tiled router GEMM + general select
+]
+
+
+@pytest.mark.parametrize("T,H,E,k,dtype,bias", ROUTE_SELECT_CASES)
+def test_route_select_matches_oracle(T, H, E, k, dtype, bias):
+    g = torch.Generator().manual_seed(T * 31 + H + E)
+    X = torch.randn(T, H, generator=g).to(dtype)
+    Wg = (torch.randn(E, H, generator=g) * (H ** -0.5)).to(dtype)
+    b = torch.randn(E, generator=g).to(dtype) if bias else None
+    d = dev()
+    xe, w, inv, off, scores = opmx().moe_route_select(X.to(d), Wg.to(d), None if b is None else b.to(d), E, k)
+    assert scores.shape == (T, E) and scores.dtype == dtype
+    ref = O.linear(X, Wg, b, out_dtype=torch.float32)
+    # one rounding of an fp32 sum; in fp32 the sum itself is only as good as its summation order
+    assert_close_ulp(scores, ref, dtype, ulps=2.0 if dtype != torch.float32 else 64.0, what="router logits")
+    rxe, rw, rinv, roff = O.moe_select(X, scores.cpu(), E, k)
+    assert torch.equal(off.cpu(), roff) and torch.equal(inv.cpu(), rinv)
+    assert torch.equal(xe.cpu().view(torch.uint8), rxe.contiguous().view(torch.uint8))
+    assert float((w.cpu().double() - rw.double()).abs().max()) <= W_TOL[dtype]
+    # the separate operators on the same inputs: same routing whenever the logits agree bit for bit
+    s2 = opmx().linear(X.to(d), Wg.to(d), None if b is None else b.to(d), H, E)
+    if torch.equal(s2, scores):
+        xe2, w2, inv2, off2 = opmx().moe_select(X.to(d), s2, E, k)
+        assert torch.equal(inv2, inv) and torch.equal(off2, off) and torch.equal(xe2, xe) and torch.equal(w2, w)
+
+
+def test_route_select_ties_go_to_the_lower_expert():
+    """Identical gate rows give identical logits for every token: all picks are ties."""
+    T, H, E, k = 8, 64, 8, 3
+    g = torch.Generator().manual_seed(5)
+    X = torch.randn(T, H, generator=g).half()
+    Wg = torch.randn(1, H, generator=g).half().repeat(E, 1)
+    d = dev()
+    xe, w, inv, off, scores = opmx().moe_route_select(X.to(d), Wg.to(d), None, E, k)
+    assert torch.equal(scores[:, :1].expand(T, E), scores)
+    assert off.cpu().tolist() == [0, T, 2 * T, 3 * T] + [3 * T] * (E - 3)
+    rxe, rw, rinv, roff = O.moe_select(X, scores.cpu(), E, k)
+    assert torch.equal(inv.cpu(), rinv) and torch.equal(xe.cpu(), rxe)
