@@ -54,6 +54,14 @@ def test_argument_validation_needs_no_device(lib):
     assert lib.opmx_moe_select(one, one, 4, 8, 8, 2, 1, one, one, one, one, None, None, 0, None) == -3      # workspace
     assert lib.opmx_moe_select(one, one, 4, 8, 8, 2, 1, one, one, one, one, None, P(8), 1 << 20, None) == -4  # align
     assert lib.opmx_moe_select(None, one, 4, 8, 8, 2, 1, one, one, one, one, None, one, 1 << 20, None) == -1
+    # router gate + select in one call: the argument checks of opmx_moe_select
+    rs = lambda *a: lib.opmx_moe_route_select(*a)
+    assert rs(one, one, None, 4, 8, 8, 9, 1, one, one, one, one, one, None, one, 1 << 20, None) == -1   # k > E
+    assert rs(one, one, None, 4, 8, 300, 2, 1, one, one, one, one, one, None, one, 1 << 20, None) == -2  # E
+    assert rs(one, one, None, 4, 8, 8, 2, 7, one, one, one, one, one, None, one, 1 << 20, None) == -2   # dtype
+    assert rs(one, one, None, 4, 8, 8, 2, 1, one, one, one, one, one, None, None, 0, None) == -3        # workspace
+    assert rs(one, None, None, 4, 8, 8, 2, 1, one, one, one, one, one, None, one, 1 << 20, None) == -1  # gate weight
+    assert rs(one, one, None, 4, 8, 8, 2, 1, None, one, one, one, one, None, one, 1 << 20, None) == -1  # scores
     assert lib.opmx_moe_column_parallel_linear(one, one, one, None, 8, 4, 64, 33, 1, 1, 0, one, None, 0, None) == -1
     assert lib.opmx_moe_column_parallel_linear(one, None, one, None, 8, 4, 64, 32, 1, 0, 0, one, None, 0, None) == -1
     assert lib.opmx_moe_row_parallel_linear(one, one, one, None, 999, 4, 64, 32, 1, 0, one, None, 0, None) == -2
