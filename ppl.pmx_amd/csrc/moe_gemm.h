@@ -115,8 +115,14 @@ __device__ __forceinline__ MTile find_mtile(const int64_t *__restrict__ off, int
     return t;
 }
 
-// Upper bound of the number of row tiles for any offsets: sum ceil(m_e/BM) <= R/BM + E.
-inline int64_t max_mtiles(int64_t R, int E, int BM) { return R / BM + E; }
+// Upper bound of the number of row tiles for any offsets: sum ceil(m_e/BM) <= R/BM + E, and
+// never more than R, as every tile holds at least one row (a single token routed to 8 of 64
+// experts: 8 tiles, not 64 -- the blocks of the others would start only to find no work).
+inline int64_t max_mtiles(int64_t R, int E, int BM)
+{
+    const int64_t bound = R / BM + E;
+    return bound < R ? bound : R;
+}
 
 // Rows outside [off[0], off[E]) belong to no expert and must read as zero
 // (MoeColumnParallelLinear.py:59 starts from torch.zeros).  Normally there are

@@ -232,3 +232,22 @@ def test_argument_errors():
         OPMX.moe_row_parallel_linear(X.cpu(), off.cpu(), W.cpu(), None, None, 1, 64, 32, True)
     Y = OPMX.moe_row_parallel_linear(X[:0], torch.zeros(2, dtype=torch.int64, device=d), W, None, None, 1, 64, 32)
     assert Y.shape == (0, 2, 32)
+
+
+@pytest.mark.parametrize("force", ["generic", "tiled", "stream"])
+def test_fewer_rows_than_experts(force):
+    """One token routed to 8 of 64 experts: 8 rows, each its own expert's only row.  The launch
+    is sized by the row count (every tile holds at least one row), not by the expert count."""
+    env = {"OPMX_MOE_GEMM": force}
+    sizes = [0] * 64
+    for e in (3, 4, 17, 30, 31, 40, 62, 63):
+        sizes[e] = 1
+    run_case("column", sizes, 256, 192, torch.bfloat16, True, env)
+    run_case("row", sizes, 128, 320, torch.float16, False, env)
+    run_case("column", sizes, 256, 2 * 96, torch.float16, True, env, swiglu=True)
+    one = [0] * 64
+    one[63] = 1                                   # a single row, for the last expert
+    run_case("row", one, 128, 64, torch.float16, True, env)
+    two = [0] * 64
+    two[0], two[63] = 2, 1                        # three rows in two tiles
+    run_case("column", two, 256, 128, torch.float16, False, env)
