@@ -15,7 +15,8 @@
 //    barrier per K-chunk;
 //  * experts with no rows produce no work, so their weights are never touched;
 //  * optional SwiGLU epilogue: a wave streams 16 gate rows and the 16 matching up rows
-//    (N/2 apart in W[e]) and combines the two accumulators in registers.
+//    (N/2 apart in W[e]) and combines the two accumulators in registers; or, for long K, a
+//    pair of waves streams one of the two each and combines through LDS after the K loop.
 // Semantics: torch_function/MoeColumnParallelLinear.py:61-67 and
 // torch_function/MoeRowParallelLinear.py:47-53 of OpenPPL/ppl.pmx.
 #include "moe_gemm.h"
@@ -32,7 +33,7 @@ template <bool NT> __device__ __forceinline__ u32x4 ld16(const char *p)
     return *reinterpret_cast<const u32x4 *>(p);
 }
 
-template <typename T, int MT, int KC, int DEPTH, bool NT, int SW, bool SG, bool PAIR>
+template <typename T, int MT, int KC, int DEPTH, bool NT, int SW, bool SG, bool PAIR, bool SGW = false>
 __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restrict__ X,
                                                                const int64_t *__restrict__ off,
                                                                const T *__restrict__ W,
@@ -42,10 +43,13 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
     // row groups per wave: SwiGLU pairs gate rows with up rows; PAIR gives a wave two adjacent
     // groups, so that a block shares its X chunk among twice the weight rows (tall row tiles,
     // where the X chunk is as large as the weight chunk)
-    static_assert(!(SG && PAIR), "one or the other");
+    // SGW: SwiGLU by wave pairs -- even waves stream gate rows, odd waves the matching up rows, one
+    // group each (the LDS footprint and chunk width of the plain form), and the pair combines its
+    // accumulators through LDS after the K loop.
+    static_assert(!(SG && PAIR) && !(SGW && (SG || PAIR)) && (!SGW || SW % 2 == 0), "one or the other");
     constexpr int NG = (SG || PAIR) ? 2 : 1;
     constexpr int WROWS = PAIR ? 32 : 16;        // output columns per wave
-    constexpr int SROWS = WROWS * SW;            // output columns per block
+    constexpr int SROWS = SGW ? 16 * SW / 2 : WROWS * SW;   // output columns per block
     constexpr int RS = KC * 2 + 16;              // LDS row stride in bytes (pad 16: conflict-free strips)
     constexpr int RPL = 512 / KC;                // W rows covered by one wave load (1 KiB)
     constexpr int NLW = 16 / RPL;                // W loads per wave per chunk
@@ -61,7 +65,7 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
     extern __shared__ __attribute__((aligned(16))) char smem[];   // [SW][WSTRIP] | [2][XBUF]
     __shared__ int64_t s_off[OPMX_MOE_MAX_EXPERTS + 1];
 
-    const int64_t ND = SG ? N / 2 : N;           // output columns; with SwiGLU W rows n and ND+n pair up
+    const int64_t ND = (SG || SGW) ? N / 2 : N;  // output columns; with SwiGLU W rows n and ND+n pair up
     zero_unowned_rows(Y, R, ND, off, E);
     const MTile mt = find_mtile(off, E, R, XM, blockIdx.y, s_off);
     if (mt.rows == 0) return;
@@ -72,7 +76,7 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
 
     // ---- this wave's 16 rows of W[e]: uniform base + per-lane byte offsets.
     // Rows past N are clamped to row N-1 (their results are masked at the store).
-    const int64_t nbase = static_cast<int64_t>(blockIdx.x) * SROWS + wave * WROWS;
+    const int64_t nbase = static_cast<int64_t>(blockIdx.x) * SROWS + (SGW ? (wave >> 1) * 16 : wave * WROWS);
     const char *wb = reinterpret_cast<const char *>(W + static_cast<int64_t>(mt.e) * N * K);
     const char *xb = reinterpret_cast<const char *>(X + mt.row0 * K);
     const int wl_row = lane / (64 / RPL);               // row inside one wave load
@@ -85,7 +89,7 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
         for (int i = 0; i < NLW; ++i) {
             const int row = i * RPL + wl_row;
             int64_t n = nbase + row + (PAIR ? g * 16 : 0);
-            n = (n < ND ? n : ND - 1) + (SG ? g * ND : 0);
+            n = (n < ND ? n : ND - 1) + (SG ? g * ND : 0) + (SGW && (wave & 1) ? ND : 0);
             wrow[g][i] = static_cast<uint32_t>(n * K * 2);
             wdst[g][i] = (g * 16 + row) * RS + wl_k * 2;
         }
@@ -186,6 +190,21 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
 #undef OPMX_STEP
 #undef OPMX_FETCH
 
+    float4_t up[MT];                 // SGW: the partner wave's accumulators (the up projection)
+    if constexpr (SGW) {
+        __syncthreads();             // every wave is done with the staging memory
+        float *exch = reinterpret_cast<float *>(smem);   // [SW/2][MT][64 lanes][4]
+        if (wave & 1) {
+#pragma unroll
+            for (int m = 0; m < MT; ++m)
+                *reinterpret_cast<float4_t *>(exch + (((wave >> 1) * MT + m) * 64 + lane) * 4) = acc[0][m];
+        }
+        __syncthreads();
+        if (wave & 1) return;
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+            up[m] = *reinterpret_cast<const float4_t *>(exch + (((wave >> 1) * MT + m) * 64 + lane) * 4);
+    }
     // acc[g][m][i]: output column nbase + fg*4 + i (W row g*ND + that), X row m*16 + fr
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
@@ -200,8 +219,8 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
                 if (n >= ND) continue;
                 float v = acc[g][m][i];
                 if (Bias) v += to_f32(Bias[static_cast<int64_t>(mt.e) * N + n]);
-                if (SG) {                          // SwiGLU.py:15-16 on the fp32 accumulators, beta = 1
-                    float u = acc[NG - 1][m][i];
+                if (SG || SGW) {                   // SwiGLU.py:15-16 on the fp32 accumulators, beta = 1
+                    float u = SGW ? up[m][i] : acc[NG - 1][m][i];
                     if (Bias) u += to_f32(Bias[static_cast<int64_t>(mt.e) * N + ND + n]);
                     v = u * v * sigmoid_fast_(v);
                 }
@@ -210,14 +229,15 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
     }
 }
 
-template <typename T, int MT, int KC, int DEPTH, bool NT, int SW, bool SG, bool PAIR = false>
+template <typename T, int MT, int KC, int DEPTH, bool NT, int SW, bool SG, bool PAIR = false, bool SGW = false>
 int stream_launch_sw(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
                      int64_t N, void *Y, hipStream_t s)
 {
-    constexpr int SROWS = (PAIR ? 32 : 16) * SW;
+    constexpr int SROWS = SGW ? 16 * SW / 2 : (PAIR ? 32 : 16) * SW;
     constexpr int RS = KC * 2 + 16;
     constexpr int smem = SW * ((SG || PAIR) ? 2 : 1) * 16 * RS + 2 * 16 * MT * RS;
-    auto kern = gemm_stream_kernel<T, MT, KC, DEPTH, NT, SW, SG, PAIR>;
+    static_assert(!SGW || (SW / 2) * MT * 1024 <= smem, "the pair exchange reuses the staging memory");
+    auto kern = gemm_stream_kernel<T, MT, KC, DEPTH, NT, SW, SG, PAIR, SGW>;
     static bool attr_done = false;
     if (!attr_done) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -225,7 +245,8 @@ int stream_launch_sw(const void *X, const int64_t *off, const void *W, const voi
             return OPMX_ERR_LAUNCH;
         attr_done = true;
     }
-    dim3 grid(static_cast<unsigned>(ceil_div(SG ? N / 2 : N, SROWS)), static_cast<unsigned>(max_mtiles(R, E, 16 * MT)));
+    dim3 grid(static_cast<unsigned>(ceil_div((SG || SGW) ? N / 2 : N, SROWS)),
+              static_cast<unsigned>(max_mtiles(R, E, 16 * MT)));
     kern<<<grid, SW * 64, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
                                      static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y));
     OPMX_LAUNCH_CHECK();
@@ -284,12 +305,12 @@ int stream_swiglu_impl(const void *X, const int64_t *off, const void *W, const v
         return K < 16 * 256 ? stream_launch<T, 1, 128, 2, true, true>(X, off, W, B, E, R, K, N, Y, s)
                             : stream_launch<T, 1, 256, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);
     if (m <= 32) {
-        // long K: the wide chunks of the plain form, in blocks of two waves (a wave holds two row
-        // groups here, so four waves with 256-wide chunks would take a CU's LDS for one block);
-        // decode T=32: 0.452 -> 0.447 ms per layer
+        // long K: SwiGLU by wave pairs, which keeps the plain form's 256-wide chunks and LDS footprint
+        // (a wave with two row groups needs twice the strip: chunks half as wide, or half the waves
+        // per CU).  Decode T=32, layer: 0.452 ms with two groups per wave, 0.442 by pairs (unfused 0.440).
         const int64_t items = ceil_div(N / 2, 64) * (R < E ? R : E);
         if (K >= 16 * 256 && items >= 512)
-            return stream_launch_sw<T, 2, 256, 2, true, 2, true>(X, off, W, B, E, R, K, N, Y, s);
+            return stream_launch_sw<T, 2, 256, 2, true, 4, false, false, true>(X, off, W, B, E, R, K, N, Y, s);
         return stream_launch<T, 2, 128, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);
     }
     if (m <= 64) return stream_launch<T, 4, 64, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);

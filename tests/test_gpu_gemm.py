@@ -194,7 +194,7 @@ def test_stream_kernel_variants(variant, dtype):
     run_case("row", [64, 40, 0, 3, 50, 33, 1, 65], 4096 + 64, 192, dtype, False, env)
     run_case("column", [1, 0, 1, 0, 0, 0, 1, 0], 1408, 2 * 128, dtype, True, env, swiglu=True)
     run_case("column", [1, 0, 1, 0, 0, 0, 1, 0], 4096, 2 * 128, dtype, False, env, swiglu=True)
-    # SwiGLU form with a long K and many weight rows: two-wave blocks with wide K chunks
+    # SwiGLU form with a long K and many weight rows: gate and up rows streamed by pairs of waves
     run_case("column", [30, 2, 17, 0, 32, 1, 25, 21], 4096, 2 * 4168, dtype, True, env, swiglu=True)
 
 
