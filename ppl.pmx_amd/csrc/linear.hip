@@ -76,6 +76,84 @@ __global__ __launch_bounds__(256) void linear_kernel(const T *__restrict__ X, co
     }
 }
 
+// Many tokens, few outputs (the router gate of a long prompt), fp16/bf16: a block takes 16 tokens
+// and all N <= 64 outputs, its NW waves split K (wave w takes the 32-wide k-steps w, w+NW, ...)
+// and feed the MFMA 16x16x32 units straight from global memory: X is read once, 64-byte pieces
+// of 16 rows per load with four steps in flight, W comes from cache.  The partial sums meet in
+// LDS and are added in wave order.  NE = 16-output tiles per token tile.
+template <typename T, int NE, int NW>
+__global__ __launch_bounds__(NW * 64) void linear_skinny_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W,
+                                                                      const T *__restrict__ B, int64_t Ttok, int64_t K,
+                                                                      int64_t N, T *__restrict__ Y)
+{
+    using frag = typename Mfma<T>::frag;
+    __shared__ __attribute__((aligned(16))) float part[NW * NE * 64 * 4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int fr = lane & 15, fg = lane >> 4;
+    const int64_t t0 = static_cast<int64_t>(blockIdx.x) * 16;
+    const int64_t trow = t0 + fr < Ttok ? t0 + fr : Ttok - 1;      // rows past the end repeat the last one
+    const T *xp = X + trow * K + fg * 8;
+    const T *wp[NE];
+#pragma unroll
+    for (int e = 0; e < NE; ++e) {
+        const int64_t n = e * 16 + fr < N ? e * 16 + fr : N - 1;
+        wp[e] = W + n * K + fg * 8;
+    }
+    float4_t acc[NE];
+#pragma unroll
+    for (int e = 0; e < NE; ++e) acc[e] = float4_t{0.f, 0.f, 0.f, 0.f};
+    const int steps = static_cast<int>(K / 32);
+    int st = wave;
+    for (; st + 3 * NW < steps; st += 4 * NW) {
+        frag b[4], a[4][NE];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            b[u] = __builtin_nontemporal_load(reinterpret_cast<const frag *>(xp + (st + NW * u) * 32));
+#pragma unroll
+            for (int e = 0; e < NE; ++e) a[u][e] = *reinterpret_cast<const frag *>(wp[e] + (st + NW * u) * 32);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int e = 0; e < NE; ++e) acc[e] = Mfma<T>::m16(a[u][e], b[u], acc[e]);
+    }
+    for (; st < steps; st += NW) {
+        const frag b = __builtin_nontemporal_load(reinterpret_cast<const frag *>(xp + st * 32));
+#pragma unroll
+        for (int e = 0; e < NE; ++e)
+            acc[e] = Mfma<T>::m16(*reinterpret_cast<const frag *>(wp[e] + st * 32), b, acc[e]);
+    }
+    // acc[e][i]: output e*16 + fg*4 + i, token t0 + fr
+#pragma unroll
+    for (int e = 0; e < NE; ++e) *reinterpret_cast<float4_t *>(part + ((wave * NE + e) * 64 + lane) * 4) = acc[e];
+    __syncthreads();
+    for (int q = threadIdx.x; q < 16 * NE * 16; q += NW * 64) {
+        const int t = q / (NE * 16), n = q % (NE * 16);
+        if (t0 + t >= Ttok || n >= N) continue;
+        const int idx = (((n >> 4) * 64) + (((n & 15) >> 2) * 16 + t)) * 4 + (n & 3);
+        float v = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) v += part[w * NE * 64 * 4 + idx];
+        if (B) v += to_f32(B[n]);
+        Y[(t0 + t) * N + n] = from_f32<T>(v);
+    }
+}
+
+template <typename T>
+int linear_skinny_mfma(const void *X, const void *W, const void *B, int64_t Ttok, int64_t K, int64_t N, void *Y,
+                       hipStream_t s)
+{
+    constexpr int NW = 8;
+    const unsigned grid = static_cast<unsigned>(ceil_div(Ttok, 16));
+    const T *x = static_cast<const T *>(X), *w = static_cast<const T *>(W), *b = static_cast<const T *>(B);
+    T *y = static_cast<T *>(Y);
+    if (N <= 16) linear_skinny_mfma_kernel<T, 1, NW><<<grid, NW * 64, 0, s>>>(x, w, b, Ttok, K, N, y);
+    else if (N <= 32) linear_skinny_mfma_kernel<T, 2, NW><<<grid, NW * 64, 0, s>>>(x, w, b, Ttok, K, N, y);
+    else linear_skinny_mfma_kernel<T, 4, NW><<<grid, NW * 64, 0, s>>>(x, w, b, Ttok, K, N, y);
+    OPMX_LAUNCH_CHECK();
+    return OPMX_OK;
+}
+
 template <typename T>
 int linear_impl(const void *X_, const void *W_, const void *B_, int64_t Ttok, int64_t K, int64_t N, void *Y_,
                 hipStream_t s)
@@ -109,6 +187,14 @@ int launch_linear(const void *X, const void *W, const void *B, int64_t T, int64_
 {
     // Many tokens: the MFMA tile kernel in dense mode (no expert_offset: one segment [0,T))
     // reads X once with 128x128 tiles instead of one pass per 8 output features.
+    // Few outputs, many tokens: the MFMA kernel that splits K over the waves of a block.  Measured
+    // against the other two (H = 4096, 8 outputs: 10 us against 19 at T = 4096, 18 against 30 at
+    // 8192, no gain below; H = 2048, 64 outputs: 12-13 us against the tile kernel's 21 from T = 512
+    // to 4096, while from 8192 tokens on the tile kernel re-reads W less and wins).
+    if ((dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16) && N <= 64 && K >= 32 && K % 32 == 0 && aligned16(X) &&
+        aligned16(W) && (N <= 8 ? T >= 4096 : (T >= 512 && (N <= 16 || T < 8192))))
+        return dtype == OPMX_DTYPE_F16 ? linear_skinny_mfma<f16>(X, W, B, T, K, N, Y, s)
+                                       : linear_skinny_mfma<bf16>(X, W, B, T, K, N, Y, s);
     if ((dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16) && T >= 512 && N > 8 && K % 64 == 0 &&
         aligned16(X) && aligned16(W) && N * K < (int64_t{1} << 31))
         return launch_gemm_tiled(X, nullptr, W, B, 1, T, K, N, dtype, OPMX_EPILOGUE_NONE, /*128x128 tiles*/ 2, Y, nullptr, 0, s);

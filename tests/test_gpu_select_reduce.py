@@ -174,7 +174,14 @@ def test_swiglu_and_silu(R, D, dtype):
                                               (8192, 4096, 8, torch.float16, False),
                                               (4096, 2048, 64, torch.bfloat16, False),
                                               (64, 1024, 8, torch.float32, True), (5, 30, 3, torch.float32, True),
-                                              (1030, 72, 20, torch.float16, True)])
+                                              (1030, 72, 20, torch.float16, True),
+                                              # many tokens, few outputs: the kernel that splits K over waves
+                                              (4097, 4096, 5, torch.float16, True),     # ragged last token tile
+                                              (600, 96, 33, torch.bfloat16, True),      # 3 k-steps for 8 waves, 3 output tiles
+                                              (513, 1024, 16, torch.float16, False),
+                                              (700, 32, 24, torch.float16, True),       # a single k-step
+                                              (2048, 4096 + 32 * 37, 48, torch.bfloat16, False),   # odd number of k-steps
+                                              (8192, 2048, 64, torch.bfloat16, True)])  # back on the tile kernel
 def test_router_linear(T, K, N, dtype, bias):
     g = torch.Generator().manual_seed(K + N)
     X = torch.randn(T, K, generator=g).to(dtype)
