@@ -195,12 +195,14 @@ __global__ __launch_bounds__(kChunk) void select_hist_kernel(const int32_t *__re
 }
 
 // ---- kernel 2: per expert exclusive scan over chunks, then offsets over experts ----
-__global__ __launch_bounds__(256) void select_scan_kernel(int32_t *__restrict__ hist, int nchunks, int E,
-                                                          int64_t R, int64_t *__restrict__ off)
+// One block; a wave scans one expert at a time (each a chain of dependent loads), so many
+// experts get a block of 16 waves.
+__global__ __launch_bounds__(1024) void select_scan_kernel(int32_t *__restrict__ hist, int nchunks, int E,
+                                                           int64_t R, int64_t *__restrict__ off)
 {
     __shared__ int total[OPMX_MOE_MAX_EXPERTS];
     const int lane = lane_id(), wave = threadIdx.x / kWave;
-    for (int e = wave; e < E; e += 256 / kWave) {
+    for (int e = wave; e < E; e += static_cast<int>(blockDim.x) / kWave) {
         int running = 0;
         for (int c0 = 0; c0 < nchunks; c0 += kWave) {
             int c = c0 + lane;
@@ -447,7 +449,7 @@ int select_impl(const void *X_, const void *scores_, int64_t Ttok, int64_t H, in
     OPMX_LAUNCH_CHECK();
     select_hist_kernel<<<nchunks, kChunk, 0, s>>>(idbuf, Ttok, E, k, hist);
     OPMX_LAUNCH_CHECK();
-    select_scan_kernel<<<1, 256, 0, s>>>(hist, nchunks, E, R, off);
+    select_scan_kernel<<<1, E > 16 ? 1024 : 256, 0, s>>>(hist, nchunks, E, R, off);
     OPMX_LAUNCH_CHECK();
     select_rank_kernel<<<nchunks, kChunk, 0, s>>>(idbuf, hist, off, Ttok, E, k, inv);
     OPMX_LAUNCH_CHECK();
