@@ -194,13 +194,43 @@ __global__ __launch_bounds__(kChunk) void select_hist_kernel(const int32_t *__re
     }
 }
 
+// Exclusive scan of count[0..E) in place, total to count[E]; called by the first wave of a block
+// (E <= 256: four experts per lane).  A single thread walking the experts costs two dependent LDS
+// round trips per expert: 6 us for 64 experts, more than the rest of the small-T kernel.
+__device__ __forceinline__ void scan_experts(int *count, int E)
+{
+    static_assert(OPMX_MOE_MAX_EXPERTS <= 4 * kWave, "four experts per lane");
+    const int lane = lane_id();
+    int v[4], tot = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int e = lane * 4 + j;
+        v[j] = e < E ? count[e] : 0;
+        tot += v[j];
+    }
+    int incl = tot;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const int o = __shfl_up(incl, d, kWave);
+        if (lane >= d) incl += o;
+    }
+    int run = incl - tot;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int e = lane * 4 + j;
+        if (e < E) count[e] = run;
+        run += v[j];
+    }
+    if (lane == kWave - 1) count[E] = incl;
+}
+
 // ---- kernel 2: per expert exclusive scan over chunks, then offsets over experts ----
 // One block; a wave scans one expert at a time (each a chain of dependent loads), so many
 // experts get a block of 16 waves.
 __global__ __launch_bounds__(1024) void select_scan_kernel(int32_t *__restrict__ hist, int nchunks, int E,
                                                            int64_t R, int64_t *__restrict__ off)
 {
-    __shared__ int total[OPMX_MOE_MAX_EXPERTS];
+    __shared__ int total[OPMX_MOE_MAX_EXPERTS + 1];
     const int lane = lane_id(), wave = threadIdx.x / kWave;
     for (int e = wave; e < E; e += static_cast<int>(blockDim.x) / kWave) {
         int running = 0;
@@ -219,14 +249,10 @@ __global__ __launch_bounds__(1024) void select_scan_kernel(int32_t *__restrict__
         if (lane == 0) total[e] = running;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        int64_t run = 0;
-        for (int e = 0; e < E; ++e) {
-            off[e] = run;                 // MoeSelect.py:54-59
-            run += total[e];
-        }
-        off[E] = R;                       // MoeSelect.py:60
-    }
+    if (threadIdx.x < kWave) scan_experts(total, E);
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += blockDim.x) off[e] = total[e];   // MoeSelect.py:54-59
+    if (threadIdx.x == 0) off[E] = R;                                      // MoeSelect.py:60
 }
 
 // ---- kernel 3: rank inside the chunk -> invert_permutation ----
@@ -344,6 +370,8 @@ __device__ __forceinline__ void router_logits_to_lds(const T *__restrict__ X, co
 
 // ---- small-T path: one launch.  Every block routes all T <= kChunk tokens
 // redundantly in LDS, then block b emits the outputs of token b and copies its row.
+// With scores == nullptr the picks are read from ids_out instead (two-launch form: the routing
+// work, T times redundant here, is what makes the one-launch form slow beyond a few tokens).
 // FUSED: the router logits are computed here as well (scores = X Wg^T + Bg, T <= kFusedTokens,
 // E <= kFusedExperts, 1024 threads) and written to `scores_out`, each block its own token's row.
 template <typename T, bool FUSED>
@@ -373,7 +401,16 @@ __global__ __launch_bounds__(1024) void select_small_kernel(const T *__restrict_
     }
     zero_bits(bits, E);
     __syncthreads();
-    for (int tl = grp; tl < Ttok; tl += ngrp) {   // whole lane groups iterate together
+    const bool picked = !FUSED && scores == nullptr;
+    if (picked) {
+        // the picks were made by select_topk_kernel (weights written there): only the bookkeeping
+        for (int q = threadIdx.x; q < Ttok * k; q += blockDim.x) {
+            const int id = ids_out[q], tl = q / k;
+            atomicOr(&bits[id * kWords + (tl >> 5)], 1u << (tl & 31));
+            if (tl == me) my_ids[q - tl * k] = id;
+        }
+    }
+    for (int tl = grp; tl < (picked ? 0 : Ttok); tl += ngrp) {   // whole lane groups iterate together
         {
             int id;
             float w;
@@ -391,15 +428,7 @@ __global__ __launch_bounds__(1024) void select_small_kernel(const T *__restrict_
     __syncthreads();
     word_prefix(bits, wordpre, count, E);
     __syncthreads();
-    if (threadIdx.x == 0) {                    // exclusive scan over experts, in place
-        int run = 0;
-        for (int e = 0; e < E; ++e) {
-            int c = count[e];
-            count[e] = run;
-            run += c;
-        }
-        count[E] = run;
-    }
+    if (threadIdx.x < kWave) scan_experts(count, E);   // exclusive scan over experts, in place
     __syncthreads();
     if (me == 0)
         for (int e = threadIdx.x; e <= E; e += blockDim.x) off[e] = count[e];
@@ -432,7 +461,11 @@ int select_impl(const void *X_, const void *scores_, int64_t Ttok, int64_t H, in
         OPMX_LAUNCH_CHECK();
         return OPMX_OK;
     }
-    if (Ttok <= kChunk && Ttok * G <= kChunk * 8) {
+    // Up to kChunk tokens.  One launch while routing every token in every block is cheap
+    // (measured: 4.8 us at T = 32 with 8 experts, 7 us at T = 4 with 64; but 14 us at T = 32 with
+    // 64 experts and 15 us at T = 256 with 8); beyond that the picks are made once per token by
+    // select_topk_kernel and the same kernel does only the bookkeeping: 6-7 us for any such T.
+    if (G == 8 ? Ttok <= 64 : (Ttok <= 16 && Ttok * G <= 512)) {
         // wide lane groups (many experts) route few tokens per wave: use a big block
         const unsigned threads = G >= 32 ? 1024 : kChunk;
         select_small_kernel<T, false><<<static_cast<unsigned>(Ttok), threads, 0, s>>>(
@@ -444,6 +477,15 @@ int select_impl(const void *X_, const void *scores_, int64_t Ttok, int64_t H, in
     char *wsb = static_cast<char *>(ws);
     int32_t *hist = reinterpret_cast<int32_t *>(wsb);
     int32_t *idbuf = ids ? ids : reinterpret_cast<int32_t *>(wsb + ceil_div(sizeof(int32_t) * nchunks * E, 256) * 256);
+    if (Ttok <= kChunk) {
+        select_topk_kernel<T><<<static_cast<unsigned>(ceil_div(Ttok, kChunk / G)), kChunk, 0, s>>>(scores, Ttok, E, k, G,
+                                                                                                   vpl, w, idbuf);
+        OPMX_LAUNCH_CHECK();
+        select_small_kernel<T, false><<<static_cast<unsigned>(Ttok), kChunk, 0, s>>>(
+            X, nullptr, static_cast<int>(Ttok), H, E, k, G, vpl, Xp, w, inv, off, idbuf, vec, nullptr, nullptr, nullptr);
+        OPMX_LAUNCH_CHECK();
+        return OPMX_OK;
+    }
     select_topk_kernel<T><<<static_cast<unsigned>(ceil_div(Ttok, kChunk / G)), kChunk, 0, s>>>(scores, Ttok, E, k, G,
                                                                                                vpl, w, idbuf);
     OPMX_LAUNCH_CHECK();

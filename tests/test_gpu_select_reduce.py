@@ -37,11 +37,17 @@ def check_select(X, s, E, k):
 
 SELECT_CASES = [
     # T, H, E, k, dtype                      path
-    (1, 64, 8, 2, torch.float16),          # single token, small path
+    (1, 64, 8, 2, torch.float16),          # single token, one launch
     (32, 4096, 8, 2, torch.float16),       # Mixtral decode
+    (64, 512, 8, 2, torch.float16),        # largest one-launch size for E=8
+    (65, 512, 8, 2, torch.float16),        # picks by the top-k kernel, bookkeeping + rows by the small kernel
     (128, 4096, 8, 2, torch.float16),
-    (256, 128, 8, 2, torch.float16),       # largest small-path size for E=8
-    (32, 2048, 64, 8, torch.bfloat16),     # fine-grained decode, small path
+    (256, 128, 8, 2, torch.float16),       # largest size of that two-launch form
+    (8, 2048, 64, 8, torch.bfloat16),      # 64 experts: one launch up to 8 tokens
+    (16, 256, 32, 4, torch.bfloat16),      # 32 experts: one launch up to 16
+    (17, 256, 32, 4, torch.bfloat16),
+    (32, 2048, 64, 8, torch.bfloat16),     # fine-grained decode, two launches
+    (200, 64, 256, 32, torch.float16),     # two launches at the limits E = 256, k = 32
     (7, 6, 5, 3, torch.float32),           # rows not 16-byte multiples: scalar copy
     (33, 40, 5, 5, torch.float32),         # k == E
     (257, 64, 8, 2, torch.float16),        # first general-path size
