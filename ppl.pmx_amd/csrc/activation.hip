@@ -5,46 +5,51 @@
 namespace opmx {
 namespace {
 
-// Y[r,i] = (g * x) * sigmoid(beta*x), x = X[r,i], g = X[r,D+i].  A thread owns one 16-byte
-// column chunk (blockIdx.x) and walks rows blockIdx.y, blockIdx.y + gridDim.y, ..., two rows per
-// step so that four loads are in flight: no index division, coalesced along the row.
-template <typename T, bool VEC>
-__global__ __launch_bounds__(256) void swiglu_kernel(const T *__restrict__ X, int64_t R, int64_t D, float beta,
-                                                     T *__restrict__ Y)
+// sigmoid for an output of type T: the accurate routine (expf and an IEEE division, some 30
+// instructions) for fp32 tensors; hardware exp2 and reciprocal (1 ulp each in fp32) where the
+// result is rounded to 16 bits anyway.  With the accurate one the 16-bit kernels are bound by the
+// vector ALUs, not by memory (-8 % on SwiGLU over [16384, 2 x 14336] fp16).
+template <typename T> __device__ __forceinline__ float sigmoid_for(float x)
 {
-    constexpr int n = VEC ? Vec16<T>::n : 1;
+    if constexpr (sizeof(T) == 2) return sigmoid_fast_(x);
+    else return sigmoidf_(x);
+}
+
+// Y[r,i] = (g * x) * sigmoid(beta*x), x = X[r,i], g = X[r,D+i].  A block takes one row of one
+// 256-chunk column strip (16 bytes per lane) and lives for that long only, so the grid (x over
+// the strips fastest, then the rows) sweeps the tensors front to back the way a plain elementwise
+// kernel does.  Measured on [16384, 2 x 14336] fp16 (1.4 GB of traffic): 224 us = 6.3 TB/s, against
+// 236 us for a plain product with the same traffic; long-lived blocks that walk the rows with a
+// stride of a few hundred ran at 4.9 TB/s, four consecutive rows per block at 5.5.
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_vec_kernel(const T *__restrict__ X, int64_t R, int64_t D, float beta,
+                                                         T *__restrict__ Y)
+{
+    constexpr int n = Vec16<T>::n;
     const int64_t c = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * n;
     if (c >= D) return;
-    const int64_t step = gridDim.y;
-    int64_t r = blockIdx.y;
-    if (VEC) {
-        for (; r + step < R; r += 2 * step) {
-            const T *p0 = X + r * 2 * D + c, *p1 = X + (r + step) * 2 * D + c;
-            Vec16<T> x0 = load16_once(p0), g0 = load16_once(p0 + D), x1 = load16_once(p1), g1 = load16_once(p1 + D), o0, o1;
+    for (int64_t r = blockIdx.y; r < R; r += gridDim.y) {
+        const Vec16<T> x = load16_once(X + r * 2 * D + c), g = load16_once(X + r * 2 * D + D + c);
+        Vec16<T> o;
 #pragma unroll
-            for (int j = 0; j < n; ++j) {
-                const float a = to_f32(x0.v[j]), b = to_f32(x1.v[j]);
-                o0.v[j] = from_f32<T>(to_f32(g0.v[j]) * a * sigmoidf_(beta * a));
-                o1.v[j] = from_f32<T>(to_f32(g1.v[j]) * b * sigmoidf_(beta * b));
-            }
-            store16(Y + r * D + c, o0);
-            store16(Y + (r + step) * D + c, o1);
+        for (int j = 0; j < n; ++j) {
+            const float a = to_f32(x.v[j]);
+            o.v[j] = from_f32<T>(to_f32(g.v[j]) * a * sigmoid_for<T>(beta * a));
         }
+        store16(Y + r * D + c, o);
     }
-    for (; r < R; r += step) {
-        const T *px = X + r * 2 * D + c;
-        if (VEC) {
-            Vec16<T> x = load16_once(px), g = load16_once(px + D), o;
-#pragma unroll
-            for (int j = 0; j < n; ++j) {
-                float xf = to_f32(x.v[j]), gf = to_f32(g.v[j]);
-                o.v[j] = from_f32<T>(gf * xf * sigmoidf_(beta * xf));
-            }
-            store16(Y + r * D + c, o);
-        } else {
-            float xf = to_f32(px[0]), gf = to_f32(px[D]);
-            Y[r * D + c] = from_f32<T>(gf * xf * sigmoidf_(beta * xf));
-        }
+}
+
+// Rows that are not whole 16-byte chunks, or unaligned tensors: one element per lane.
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_scalar_kernel(const T *__restrict__ X, int64_t R, int64_t D, float beta,
+                                                            T *__restrict__ Y)
+{
+    const int64_t c = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (c >= D) return;
+    for (int64_t r = blockIdx.y; r < R; r += gridDim.y) {
+        const float xf = to_f32(X[r * 2 * D + c]), gf = to_f32(X[r * 2 * D + D + c]);
+        Y[r * D + c] = from_f32<T>(gf * xf * sigmoid_for<T>(beta * xf));
     }
 }
 
@@ -62,13 +67,13 @@ __global__ __launch_bounds__(256) void silu_kernel(const T *__restrict__ X, cons
 #pragma unroll
             for (int j = 0; j < n; ++j) {
                 float xf = to_f32(x.v[j]);
-                float y = xf * sigmoidf_(xf);
+                float y = xf * sigmoid_for<T>(xf);
                 o.v[j] = from_f32<T>(gate ? to_f32(g.v[j]) * y : y);
             }
             store16(Y + i * n, o);
         } else {
             float xf = to_f32(X[i]);
-            float y = xf * sigmoidf_(xf);
+            float y = xf * sigmoid_for<T>(xf);
             Y[i] = from_f32<T>(gate ? to_f32(gate[i]) * y : y);
         }
     }
@@ -85,17 +90,12 @@ template <typename T> int swiglu_impl(const void *X, int64_t R, int64_t D, float
     if (R == 0 || D == 0) return OPMX_OK;
     constexpr int n = Vec16<T>::n;
     const bool vec = D % n == 0 && aligned16(X) && aligned16(Y);
-    // columns over x; rows over y, as many row lanes as it takes to have ~16 blocks per CU
     const int64_t chunks = vec ? D / n : D;
-    const unsigned gx = static_cast<unsigned>(ceil_div(chunks, 256));
-    int64_t gy = ceil_div(4096, gx);
-    if (gy > R) gy = R;
-    if (gy > 65535) gy = 65535;
-    const dim3 grid(gx, static_cast<unsigned>(gy));
+    const dim3 grid(static_cast<unsigned>(ceil_div(chunks, 256)), static_cast<unsigned>(R < 65535 ? R : 65535));
     if (vec)
-        swiglu_kernel<T, true><<<grid, 256, 0, s>>>(static_cast<const T *>(X), R, D, beta, static_cast<T *>(Y));
+        swiglu_vec_kernel<T><<<grid, 256, 0, s>>>(static_cast<const T *>(X), R, D, beta, static_cast<T *>(Y));
     else
-        swiglu_kernel<T, false><<<grid, 256, 0, s>>>(static_cast<const T *>(X), R, D, beta, static_cast<T *>(Y));
+        swiglu_scalar_kernel<T><<<grid, 256, 0, s>>>(static_cast<const T *>(X), R, D, beta, static_cast<T *>(Y));
     OPMX_LAUNCH_CHECK();
     return OPMX_OK;
 }
