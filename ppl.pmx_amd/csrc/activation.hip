@@ -79,10 +79,12 @@ __global__ __launch_bounds__(256) void silu_kernel(const T *__restrict__ X, cons
     }
 }
 
+// One 256-lane block per 256 work items (the kernel strides on only past 2^31 - 1 blocks): short
+// blocks in address order stream faster than a few long-lived ones (see swiglu_vec_kernel).
 inline unsigned grid_for(int64_t work_items)
 {
-    int64_t b = ceil_div(work_items, 256);
-    return static_cast<unsigned>(b < 1 ? 1 : (b > 8192 ? 8192 : b));
+    const int64_t b = ceil_div(work_items, 256), most = (int64_t{1} << 31) - 1;
+    return static_cast<unsigned>(b < 1 ? 1 : (b > most ? most : b));
 }
 
 template <typename T> int swiglu_impl(const void *X, int64_t R, int64_t D, float beta, void *Y, hipStream_t s)
