@@ -24,7 +24,8 @@ already resident in HBM.  Prints ONE JSON line:
 
 Workloads (--workload): decode-T{1,8,32,128} and prefill-T{2048,8192} at the
 Mixtral-8x7B shape (fp16), fine-T{32,4096} (64 experts, top-8, bf16),
-8x22b-T{16,4096}.  Default: decode-T32, the configuration the metric is quoted on.
+8x22b-T{16,4096}; e128-T<n> / e256-T<n>: 128 / 256 small experts (bf16).  Any T is accepted.
+Default: decode-T32, the configuration the metric is quoted on.
 """
 import argparse
 import json
@@ -54,6 +55,9 @@ SHAPES = {
     "prefill": dict(H=4096, E=8, k=2, I=14336, dtype="float16", skew=1.5, name="mixtral-8x7b"),
     "fine": dict(H=2048, E=64, k=8, I=1408, dtype="bfloat16", skew=0.0, name="fine-grained-64x8"),
     "8x22b": dict(H=6144, E=8, k=2, I=16384, dtype="float16", skew=0.0, name="mixtral-8x22b-shape"),
+    # further shapes (not part of the reference's configurations): many small experts
+    "e128": dict(H=2048, E=128, k=8, I=768, dtype="bfloat16", skew=0.0, name="128-experts-top8-ffn768"),
+    "e256": dict(H=7168, E=256, k=8, I=2048, dtype="bfloat16", skew=0.0, name="256-experts-top8-ffn2048"),
 }
 
 

@@ -71,47 +71,73 @@ struct MTile {
     int64_t row0;
 };
 
-// Copies expert_offset into LDS (clamped to a non-decreasing sequence inside
-// [0, R], so a corrupt offset can never send a store outside Y) and finds the
-// `tile`-th row tile of height BM in expert order.  s_off needs E+1 entries.
-// Every thread of the block must call it; it contains block barriers.
-__device__ __forceinline__ MTile find_mtile(const int64_t *__restrict__ off, int E, int64_t R, int BM,
-                                            int64_t tile, int64_t *s_off)
+// Finds the `tile`-th row tile of height BM in expert order, straight from expert_offset.
+// Every wave works it out for itself, four experts per lane (E <= 256): tile counts per expert,
+// a prefix sum over the lanes, one ballot for the lane that owns the tile -- no LDS, no block
+// barrier, and no walk over the experts by every thread (with 256 experts that walk took longer
+// than a short block's whole K loop).  Offsets are clamped into [0, R] and a segment that ends
+// before it starts counts as empty, so a corrupt offset can never send a store outside Y.
+// Every thread of the block must call it (whole waves, converged).
+__device__ __forceinline__ MTile find_mtile(const int64_t *__restrict__ off, int E, int64_t R, int BM, int64_t tile)
 {
-    if (off == nullptr) {               // dense GEMM: one "expert" owns rows [0, R)
-        MTile d;
-        d.e = 0;
-        d.row0 = tile * BM;
-        const int64_t left = R - d.row0;
-        d.rows = left <= 0 ? 0 : static_cast<int>(left < BM ? left : BM);
-        return d;
-    }
-    for (int i = threadIdx.x; i <= E; i += blockDim.x) {
-        int64_t v = off[i];
-        s_off[i] = v < 0 ? 0 : (v > R ? R : v);
-    }
-    __syncthreads();
+    static_assert(OPMX_MOE_MAX_EXPERTS <= 4 * kWave, "four experts per lane");
     MTile t;
     t.e = 0;
     t.rows = 0;
     t.row0 = 0;
-    int64_t prev = s_off[0];
-    for (int e = 0; e < E; ++e) {
-        int64_t lo = prev, hi = s_off[e + 1];
-        if (hi < lo) hi = lo;
-        const int64_t nt = (hi - lo + BM - 1) / BM;
-        if (tile < nt) {
-            // block-uniform by construction; say so to the compiler (scalar registers)
-            const int64_t row0 = lo + tile * BM, left = hi - row0;
-            t.e = __builtin_amdgcn_readfirstlane(e);
-            t.row0 = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0 >> 32))) << 32) |
-                     static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0)));
-            t.rows = __builtin_amdgcn_readfirstlane(static_cast<int>(left < BM ? left : BM));
-            return t;
-        }
-        tile -= nt;
-        prev = hi;
+    if (off == nullptr) {               // dense GEMM: one "expert" owns rows [0, R)
+        t.row0 = tile * BM;
+        const int64_t left = R - t.row0;
+        t.rows = left <= 0 ? 0 : static_cast<int>(left < BM ? left : BM);
+        return t;
     }
+    const int lane = threadIdx.x & (kWave - 1);
+    int64_t o[5];
+#pragma unroll
+    for (int j = 0; j < 5; ++j) {
+        const int idx = lane * 4 + j;
+        const int64_t v = off[idx < E ? idx : E];
+        o[j] = v < 0 ? 0 : (v > R ? R : v);
+    }
+    int nt[4], tot = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int64_t rows = o[j + 1] - o[j];
+        nt[j] = (lane * 4 + j < E && rows > 0) ? static_cast<int>((rows + BM - 1) / BM) : 0;
+        tot += nt[j];
+    }
+    int incl = tot;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const int up = __shfl_up(incl, d, kWave);
+        if (lane >= d) incl += up;
+    }
+    const int excl = incl - tot;
+    const int want = tile < (int64_t{1} << 31) ? static_cast<int>(tile) : 0x7fffffff;
+    const uint64_t owner = __ballot(want >= excl && want < incl);
+    if (owner == 0) return t;           // past the last tile (uniform)
+    const int src = __ffsll(static_cast<long long>(owner)) - 1;
+    // the owning lane picks the expert among its four
+    int e_local = 3, before = excl + nt[0] + nt[1] + nt[2];
+    if (want < excl + nt[0]) {
+        e_local = 0;
+        before = excl;
+    } else if (want < excl + nt[0] + nt[1]) {
+        e_local = 1;
+        before = excl + nt[0];
+    } else if (want < excl + nt[0] + nt[1] + nt[2]) {
+        e_local = 2;
+        before = excl + nt[0] + nt[1];
+    }
+    const int64_t lo = e_local == 0 ? o[0] : e_local == 1 ? o[1] : e_local == 2 ? o[2] : o[3];
+    const int64_t hi = e_local == 0 ? o[1] : e_local == 1 ? o[2] : e_local == 2 ? o[3] : o[4];
+    const int64_t row0 = lo + static_cast<int64_t>(want - before) * BM, left = hi - row0;
+    const int rows = static_cast<int>(left < BM ? left : BM);
+    // block-uniform by construction; say so to the compiler (scalar registers)
+    t.e = __builtin_amdgcn_readlane(lane * 4 + e_local, src);
+    t.row0 = (static_cast<int64_t>(__builtin_amdgcn_readlane(static_cast<int>(row0 >> 32), src)) << 32) |
+             static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(row0), src));
+    t.rows = __builtin_amdgcn_readlane(rows, src);
     return t;
 }
 

@@ -17,12 +17,11 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T *__restrict__
                                                            int E, int64_t R, int64_t K, int64_t N,
                                                            T *__restrict__ Y)
 {
-    __shared__ int64_t s_off[OPMX_MOE_MAX_EXPERTS + 1];
     __shared__ float As[GK][GB + 4];
     __shared__ float Bs[SWIGLU ? 2 : 1][GK][GB + 4];
     const int64_t ncols = SWIGLU ? N / 2 : N;      // output columns
     zero_unowned_rows(Y, R, ncols, off, E);
-    const MTile mt = find_mtile(off, E, R, GB, blockIdx.y, s_off);
+    const MTile mt = find_mtile(off, E, R, GB, blockIdx.y);
     if (mt.rows == 0) return;
     const int64_t n0 = static_cast<int64_t>(blockIdx.x) * GB;
     const T *We = W + static_cast<int64_t>(mt.e) * N * K;

@@ -63,11 +63,10 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
     using frag = typename Mfma<T>::frag;
 
     extern __shared__ __attribute__((aligned(16))) char smem[];   // [SW][WSTRIP] | [2][XBUF]
-    __shared__ int64_t s_off[OPMX_MOE_MAX_EXPERTS + 1];
 
     const int64_t ND = (SG || SGW) ? N / 2 : N;  // output columns; with SwiGLU W rows n and ND+n pair up
     zero_unowned_rows(Y, R, ND, off, E);
-    const MTile mt = find_mtile(off, E, R, XM, blockIdx.y, s_off);
+    const MTile mt = find_mtile(off, E, R, XM, blockIdx.y);
     if (mt.rows == 0) return;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
