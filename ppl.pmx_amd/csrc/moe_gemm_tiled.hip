@@ -35,32 +35,75 @@ constexpr int CH = ROWB / 16;          // 16-byte chunks per row (8)
 // column land in sixteen different 16-byte bank groups (conflict-free b128 fragment reads).
 __device__ __forceinline__ int lds_off(int row, int chunk) { return row * ROWB + ((chunk ^ ((row >> 1) & 7)) << 4); }
 
-// Clamped copy of expert_offset in LDS (values forced into a non-decreasing sequence inside
-// [0, R] when read, so a corrupt offset can never send a store outside Y).  Nothing to do for a
-// dense GEMM (off == nullptr).  Every thread must call it: it contains a block barrier.
-__device__ __forceinline__ void stage_offsets(const int64_t *__restrict__ off, int E, int64_t R, int64_t *s_off)
+// What a workgroup knows about the experts, in LDS: the offsets clamped into [0, R] (a corrupt
+// offset can never send a store outside Y; a segment that ends before it starts counts as empty)
+// and the running number of row tiles in front of every expert.  Looking a tile up is then a
+// search in `pref`, done by the lanes of a wave together (find_expert) instead of a walk over the
+// experts by every thread: with 64 experts that walk cost a microsecond per tile, with 256 four.
+struct ExpertTable {
+    int64_t off[OPMX_MOE_MAX_EXPERTS + 1];
+    int pref[OPMX_MOE_MAX_EXPERTS + 4];     // pref[e] = row tiles of experts < e; pref[E ... 256] = all of them
+};
+
+// Fills the table for row tiles of height BM.  Nothing to do for a dense GEMM (off == nullptr).
+// Every thread must call it: it contains block barriers.
+__device__ __forceinline__ void stage_offsets(const int64_t *__restrict__ off, int E, int64_t R, int BM, ExpertTable &tab)
 {
+    static_assert(OPMX_MOE_MAX_EXPERTS <= 4 * 64, "four experts per lane");
     if (off == nullptr) return;
     for (int i = threadIdx.x; i <= E; i += blockDim.x) {
         const int64_t v = off[i];
-        s_off[i] = v < 0 ? 0 : (v > R ? R : v);
+        tab.off[i] = v < 0 ? 0 : (v > R ? R : v);
+    }
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        const int lane = threadIdx.x, sh = 31 - __builtin_clz(BM);    // BM is a power of two
+        int m[4], tot = 0;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int e = lane * 4 + q;
+            const int64_t rows = e < E ? tab.off[e + 1] - tab.off[e] : 0;
+            m[q] = rows > 0 ? static_cast<int>((rows + BM - 1) >> sh) : 0;
+            tot += m[q];
+        }
+        int incl = tot;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int up = __shfl_up(incl, d, 64);
+            if (lane >= d) incl += up;
+        }
+        int run = incl - tot;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            tab.pref[lane * 4 + q] = run;
+            run += m[q];
+        }
+        if (lane == 63) tab.pref[256] = incl;
     }
     __syncthreads();
 }
 
 // Number of row tiles of height BM over all experts: sum of ceil(rows_e / BM).
-__device__ __forceinline__ int count_mtiles(bool grouped, const int64_t *s_off, int E, int64_t R, int BM)
+__device__ __forceinline__ int count_mtiles(bool grouped, const ExpertTable &tab, int E, int64_t R, int BM)
 {
     const int sh = 31 - __builtin_clz(BM);       // BM is a power of two: shifts, not 64-bit divisions
     if (!grouped) return static_cast<int>((R + BM - 1) >> sh);
-    int64_t total = 0, prev = s_off[0];
-    for (int e = 0; e < E; ++e) {
-        int64_t hi = s_off[e + 1];
-        if (hi < prev) hi = prev;
-        total += (hi - prev + BM - 1) >> sh;
-        prev = hi;
-    }
-    return __builtin_amdgcn_readfirstlane(static_cast<int>(total));
+    return __builtin_amdgcn_readfirstlane(tab.pref[256]);
+}
+
+// The expert that owns row tile `tile_m` (counted over all experts in expert order), or -1.
+// Whole waves, converged; the answer is wave-uniform.
+__device__ __forceinline__ int find_expert(int tile_m, const ExpertTable &tab)
+{
+    const int lane = threadIdx.x & 63;
+    int p[5];
+#pragma unroll
+    for (int q = 0; q < 5; ++q) p[q] = tab.pref[lane * 4 + q];
+    const uint64_t owner = __ballot(tile_m >= p[0] && tile_m < p[4]);
+    if (tile_m < 0 || owner == 0) return -1;
+    const int src = __ffsll(static_cast<long long>(owner)) - 1;
+    const int q = tile_m < p[1] ? 0 : (tile_m < p[2] ? 1 : (tile_m < p[3] ? 2 : 3));
+    return __builtin_amdgcn_readlane(lane * 4 + q, src);
 }
 
 // Linear tile id -> (row tile, column tile) over the row tiles of all experts strung together;
@@ -99,9 +142,9 @@ __device__ __forceinline__ void map_tile(int lin, int gnx, int mtiles, int ntile
 }
 
 // Row tile tile_m (counted over all experts in expert order) -> expert and row range.
-// mt.rows == 0 when there is no such tile.  s_off: see stage_offsets (unused when `grouped` is
+// mt.rows == 0 when there is no such tile.  tab: see stage_offsets (unused when `grouped` is
 // false: one expert owns [0, R)).
-__device__ __forceinline__ void row_tile(int tile_m, bool grouped, const int64_t *s_off, int E, int64_t R, int BM,
+__device__ __forceinline__ void row_tile(int tile_m, bool grouped, const ExpertTable &tab, int E, int64_t R, int BM,
                                          MTile &mt)
 {
     mt.e = 0;
@@ -114,24 +157,14 @@ __device__ __forceinline__ void row_tile(int tile_m, bool grouped, const int64_t
         mt.rows = left <= 0 ? 0 : static_cast<int>(left < BM ? left : BM);
         return;
     }
-    const int sh = 31 - __builtin_clz(BM);       // BM is a power of two
-    int64_t tile = tile_m, prev = s_off[0];
-    for (int e = 0; e < E; ++e) {
-        int64_t hi = s_off[e + 1];
-        if (hi < prev) hi = prev;
-        const int64_t nt = (hi - prev + BM - 1) >> sh;
-        if (tile < nt) {
-            // block-uniform by construction; say so to the compiler (scalar registers)
-            const int64_t row0 = prev + tile * BM, left = hi - row0;
-            mt.e = __builtin_amdgcn_readfirstlane(e);
-            mt.row0 = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0 >> 32))) << 32) |
-                      static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0)));
-            mt.rows = __builtin_amdgcn_readfirstlane(static_cast<int>(left < BM ? left : BM));
-            return;
-        }
-        tile -= nt;
-        prev = hi;
-    }
+    const int e = find_expert(tile_m, tab);
+    if (e < 0) return;
+    const int64_t row0 = tab.off[e] + static_cast<int64_t>(tile_m - tab.pref[e]) * BM, left = tab.off[e + 1] - row0;
+    // block-uniform by construction; say so to the compiler (scalar registers)
+    mt.e = e;
+    mt.row0 = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0 >> 32))) << 32) |
+              static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0)));
+    mt.rows = __builtin_amdgcn_readfirstlane(static_cast<int>(left < BM ? left : BM));
 }
 
 // Expert-major order (gnx = 8; ntiles_n % 8 == 0).  The orders above lay their XCD sub-blocks
@@ -151,7 +184,7 @@ __device__ __forceinline__ void row_tile(int tile_m, bool grouped, const int64_t
 //    (h = 8, or what is left): each W-tile is shared by h of them, each X-tile by 32/h.
 // Every XCD gets exactly an eighth of every expert, and the ids [0, sum m_e * ntiles_n) are
 // exactly the tiles.
-__device__ __forceinline__ void locate_expert_major(int64_t lin, bool grouped, const int64_t *s_off, int E, int64_t R,
+__device__ __forceinline__ void locate_expert_major(int64_t lin, bool grouped, const ExpertTable &tab, int E, int64_t R,
                                                     int BM, int ntiles_n, MTile &mt, int &tile_n)
 {
     mt.e = 0;
@@ -160,45 +193,51 @@ __device__ __forceinline__ void locate_expert_major(int64_t lin, bool grouped, c
     tile_n = 0;
     const int sh = 31 - __builtin_clz(BM);
     const uint32_t C = static_cast<uint32_t>(ntiles_n) >> 3;
-    int64_t base = 0, prev = grouped ? s_off[0] : 0;
-    const int experts = grouped ? E : 1;
-    for (int e = 0; e < experts; ++e) {
-        int64_t hi = grouped ? s_off[e + 1] : R;
-        if (hi < prev) hi = prev;
-        const uint32_t m = static_cast<uint32_t>((hi - prev + BM - 1) >> sh);
-        const int64_t n = static_cast<int64_t>(m) * ntiles_n;
-        if (lin < base + n) {
-            uint32_t l = static_cast<uint32_t>(lin - base), row, col;
-            const uint32_t band = 16u * static_cast<uint32_t>(ntiles_n), bands = m >> 4;
-            if (l < bands * band) {
-                const uint32_t b = l / band, l2 = l - b * band, xcd = l2 & 7, s = l2 >> 3;
-                row = b * 16 + (xcd >> 2) * 8 + (s & 7);
-                col = (xcd & 3) * (2 * C) + (s >> 3);
-            } else {
-                l -= bands * band;
-                const uint32_t mr = m - 16 * bands, xcd = l & 7, s = l >> 3;   // s in [0, mr*C)
-                const uint32_t full = mr >> 3, per_group = 8 * C;
-                uint32_t rg = s / per_group, h = 8;
-                if (rg >= full) {
-                    rg = full;
-                    h = mr - 8 * full;
-                }
-                const uint32_t t = s - rg * per_group, c = t / h;
-                row = 16 * bands + rg * 8 + (t - c * h);
-                col = xcd * C + c;
-            }
-            const int64_t row0 = prev + static_cast<int64_t>(row) * BM, left = hi - row0;
-            // block-uniform by construction; say so to the compiler (scalar registers)
-            tile_n = __builtin_amdgcn_readfirstlane(static_cast<int>(col));
-            mt.e = __builtin_amdgcn_readfirstlane(e);
-            mt.row0 = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0 >> 32))) << 32) |
-                      static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0)));
-            mt.rows = __builtin_amdgcn_readfirstlane(static_cast<int>(left < BM ? left : BM));
-            return;
-        }
-        base += n;
-        prev = hi;
+    // expert e owns the ids [pref[e] * ntiles_n, pref[e+1] * ntiles_n): its row tiles times all columns
+    int e = 0;
+    uint32_t m, l;
+    int64_t prev = 0, hi = R;
+    if (grouped) {
+        if (lin >= (int64_t{1} << 31)) return;
+        const uint32_t g = static_cast<uint32_t>(lin) / static_cast<uint32_t>(ntiles_n);
+        e = find_expert(static_cast<int>(g), tab);
+        if (e < 0) return;
+        const uint32_t first = static_cast<uint32_t>(tab.pref[e]);
+        m = static_cast<uint32_t>(tab.pref[e + 1]) - first;
+        l = static_cast<uint32_t>(lin) - first * static_cast<uint32_t>(ntiles_n);
+        prev = tab.off[e];
+        hi = tab.off[e + 1];
+    } else {
+        m = static_cast<uint32_t>((R + BM - 1) >> sh);
+        if (lin >= static_cast<int64_t>(m) * ntiles_n) return;
+        l = static_cast<uint32_t>(lin);
     }
+    uint32_t row, col;
+    const uint32_t band = 16u * static_cast<uint32_t>(ntiles_n), bands = m >> 4;
+    if (l < bands * band) {
+        const uint32_t b = l / band, l2 = l - b * band, xcd = l2 & 7, s = l2 >> 3;
+        row = b * 16 + (xcd >> 2) * 8 + (s & 7);
+        col = (xcd & 3) * (2 * C) + (s >> 3);
+    } else {
+        l -= bands * band;
+        const uint32_t mr = m - 16 * bands, xcd = l & 7, s = l >> 3;   // s in [0, mr*C)
+        const uint32_t full = mr >> 3, per_group = 8 * C;
+        uint32_t rg = s / per_group, h = 8;
+        if (rg >= full) {
+            rg = full;
+            h = mr - 8 * full;
+        }
+        const uint32_t t = s - rg * per_group, c = t / h;
+        row = 16 * bands + rg * 8 + (t - c * h);
+        col = xcd * C + c;
+    }
+    const int64_t row0 = prev + static_cast<int64_t>(row) * BM, left = hi - row0;
+    // block-uniform by construction; say so to the compiler (scalar registers)
+    tile_n = __builtin_amdgcn_readfirstlane(static_cast<int>(col));
+    mt.e = __builtin_amdgcn_readfirstlane(e);
+    mt.row0 = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0 >> 32))) << 32) |
+              static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0)));
+    mt.rows = __builtin_amdgcn_readfirstlane(static_cast<int>(left < BM ? left : BM));
 }
 
 // Row-partition order (gnx = 16), for column-tile counts that do not divide by 8 (11 column tiles
@@ -225,7 +264,7 @@ __device__ __forceinline__ void map_row_partition(int64_t lin, int mtiles, int n
 
 // Linear tile id -> tile, in whichever order gnx names.  mt.rows == 0: the id names no work.
 __device__ __forceinline__ void locate_any(int64_t lin, int gnx, int mtiles, int ntiles_n, bool grouped,
-                                           const int64_t *s_off, int E, int64_t R, int BM, MTile &mt, int &tile_n)
+                                           const ExpertTable &s_off, int E, int64_t R, int BM, MTile &mt, int &tile_n)
 {
     if (gnx == 8) {
         locate_expert_major(lin, grouped, s_off, E, R, BM, ntiles_n, mt, tile_n);
@@ -428,12 +467,12 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
     using frag = typename Mfma<T>::frag;
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    __shared__ int64_t s_off[OPMX_MOE_MAX_EXPERTS + 1];
+    __shared__ ExpertTable s_off;
 
     const int64_t ncols = SWIGLU ? N / 2 : N;
     zero_unowned_rows(Y, R, ncols, off, E);
 
-    stage_offsets(off, E, R, s_off);
+    stage_offsets(off, E, R, BM, s_off);
     MTile mt;
     int tile_n;
     locate_any(blockIdx.x, gnx, count_mtiles(off != nullptr, s_off, E, R, BM), ntiles_n, off != nullptr, s_off, E, R,
@@ -792,12 +831,12 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
     using frag = typename Mfma<T>::frag;
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    __shared__ int64_t s_off[OPMX_MOE_MAX_EXPERTS + 1];
+    __shared__ ExpertTable s_off;
 
     __shared__ int s_arrivals;
     const int64_t ncols = SWIGLU ? N / 2 : N;
     if (!SK) zero_unowned_rows(Y, R, ncols, off, E);
-    stage_offsets(off, E, R, s_off);
+    stage_offsets(off, E, R, BM, s_off);
     const int mtiles = count_mtiles(off != nullptr, s_off, E, R, BM);
     const int nk = static_cast<int>(K / BK);
     const int krot = k_rotation(nk);
@@ -1147,11 +1186,11 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
     using frag = typename Mfma<T>::frag;
 
     extern __shared__ __attribute__((aligned(16))) char smem[];      // two stages, then NW staging regions
-    __shared__ int64_t s_off[OPMX_MOE_MAX_EXPERTS + 1];
+    __shared__ ExpertTable s_off;
 
     const int64_t ncols = SWIGLU ? N / 2 : N;
     zero_unowned_rows(Y, R, ncols, off, E);
-    stage_offsets(off, E, R, s_off);
+    stage_offsets(off, E, R, BM, s_off);
     const int mtiles = count_mtiles(off != nullptr, s_off, E, R, BM);
     const int nk = static_cast<int>(K / BK);
     const int krot = k_rotation(nk);
