@@ -132,6 +132,49 @@ class MoeFeedForward(nn.Module):
         return used
 
 
+class GraphedMoeFeedForward(nn.Module):
+    """Replays a ``MoeFeedForward`` from HIP graphs, one per input shape (no counterpart in the
+    reference, whose model runs eagerly under ``torch.inference_mode``, ``Model.py:318``).
+
+    With few tokens the six operators take a few microseconds of GPU time each and the host's launch
+    path sets the pace; a serving loop captures the layer once per batch size and replays it.  The
+    first call with a new shape runs the block once eagerly (kernel attributes are set on first
+    launch), captures it on a side stream into static buffers, and every call copies the input in,
+    replays, and returns the static output -- valid until the next call with the same shape; clone
+    it to keep it.  ``max_graphs`` bounds the number of shapes kept (oldest dropped first).
+    """
+
+    def __init__(self, block: MoeFeedForward, max_graphs: int = 16):
+        super().__init__()
+        self.block = block
+        self.max_graphs = max_graphs
+        self._graphs = {}          # (shape, dtype, device) -> (graph, static input, static output)
+
+    @torch.inference_mode()
+    def forward(self, x):
+        if torch.onnx.is_in_onnx_export() or not x.is_cuda:
+            return self.block(x)
+        key = (tuple(x.shape), x.dtype, x.device)
+        entry = self._graphs.get(key)
+        if entry is None:
+            static_x = x.clone()
+            side = torch.cuda.Stream(device=x.device)
+            side.wait_stream(torch.cuda.current_stream(x.device))
+            with torch.cuda.stream(side):
+                self.block(static_x)
+            torch.cuda.current_stream(x.device).wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                static_out = self.block(static_x)
+            if len(self._graphs) >= self.max_graphs:
+                self._graphs.pop(next(iter(self._graphs)))
+            entry = self._graphs[key] = (graph, static_x, static_out)
+        graph, static_x, static_out = entry
+        static_x.copy_(x)
+        graph.replay()
+        return static_out
+
+
 def load_opmx_moe_block(path, layer_id: int, num_experts_per_token: int, fused_ffn_glu: bool = True,
                         dtype=None, device=None, fuse_swiglu_epilogue: bool = False, fuse_router_select: bool = False):
     """Builds the MoE block of layer ``layer_id`` from an OPMX Mixtral ``.pth`` checkpoint.

@@ -51,3 +51,22 @@ def test_captured_layer_replays_the_eager_result(T, H, I, E, k, dtype, fuse, rou
                 torch.cuda.synchronize()
                 assert torch.equal(got, want), (rep, float((got.float() - want.float()).abs().max()))
                 assert other.shape == want.shape
+
+
+def test_graphed_block_matches_the_eager_block():
+    """GraphedMoeFeedForward: one graph per input shape, results equal to the eager block bit for
+    bit, shapes interleaved, the oldest graph dropped when the bound is reached."""
+    from model_zoo.mixtral.modeling.dynamic_batching.Model import GraphedMoeFeedForward
+    H, I, E, k, dtype = 512, 1408, 8, 2, torch.float16
+    (x, Wg, wu, w2), _ = gpu_inputs(64, H, E, I, dtype, seed=5)
+    block = build_layer(H, I, E, k, dtype, Wg, wu, w2)
+    graphed = GraphedMoeFeedForward(block, max_graphs=2)
+    gen = torch.Generator(device="cuda").manual_seed(2)
+    with torch.inference_mode():
+        for T in (1, 32, 1, 64, 32, 1):               # three shapes through a bound of two
+            xi = torch.randn(T, H, generator=gen, device=dev()).to(dtype)
+            want = block(xi)
+            got = graphed(xi).clone()
+            torch.cuda.synchronize()
+            assert torch.equal(got, want), T
+            assert len(graphed._graphs) <= 2
