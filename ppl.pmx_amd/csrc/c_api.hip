@@ -76,7 +76,8 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
     else if (force == 1) choice = 1;
     else if (mfma_ok && stream_ws && hint <= kStreamMaxRowsPerExpert) choice = 3;
     else if (tiled_ok) choice = 2;
-    else choice = 1;
+    else if (mfma_ok && stream_ws) choice = 3;   // K a multiple of 8 but not of 64: 128-row tiles of the stream kernel
+    else choice = 1;                             // (MFMA, weights re-read per row tile) rather than the FMA fallback
 
     if (choice == 3)
         return launch_gemm_stream(X, off, W, B, E, R, K, N, dtype, epilogue, hint,

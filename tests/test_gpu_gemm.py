@@ -204,6 +204,10 @@ def test_automatic_selection_and_hint(dtype):
     run_case("column", [10, 6, 0, 16, 8, 8, 9, 7], 512, 256, dtype, False, lead3=True)
     run_case("column", [700, 6, 0, 16, 800, 8, 90, 428], 512, 256, dtype, False, lead3=True)
     run_case("row", [700, 6, 0, 16, 800, 8, 90, 428], 512, 256, dtype, True)
+    if dtype != torch.float32:
+        # K a multiple of 8 but not of 64 with many rows: the stream kernel's 128-row tiles, not the FMA fallback
+        run_case("column", [700, 6, 0, 16, 800, 8, 90, 428], 520, 256, dtype, True)
+        run_case("row", [700, 6, 0, 16, 800, 8, 90, 428], 1000, 192, dtype, False)
 
 
 @pytest.mark.parametrize("force", ["generic", "tiled", "stream"])
