@@ -93,10 +93,11 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_mfma_kernel(const T *__
     const int64_t t0 = static_cast<int64_t>(blockIdx.x) * 16;
     const int64_t trow = t0 + fr < Ttok ? t0 + fr : Ttok - 1;      // rows past the end repeat the last one
     const T *xp = X + trow * K + fg * 8;
+    const int64_t n0 = static_cast<int64_t>(blockIdx.y) * (NE * 16);   // this block's outputs: [n0, n0 + 16 NE)
     const T *wp[NE];
 #pragma unroll
     for (int e = 0; e < NE; ++e) {
-        const int64_t n = e * 16 + fr < N ? e * 16 + fr : N - 1;
+        const int64_t n = n0 + e * 16 + fr < N ? n0 + e * 16 + fr : N - 1;
         wp[e] = W + n * K + fg * 8;
     }
     float4_t acc[NE];
@@ -129,13 +130,13 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_mfma_kernel(const T *__
     __syncthreads();
     for (int q = threadIdx.x; q < 16 * NE * 16; q += NW * 64) {
         const int t = q / (NE * 16), n = q % (NE * 16);
-        if (t0 + t >= Ttok || n >= N) continue;
+        if (t0 + t >= Ttok || n0 + n >= N) continue;
         const int idx = (((n >> 4) * 64) + (((n & 15) >> 2) * 16 + t)) * 4 + (n & 3);
         float v = 0.0f;
 #pragma unroll
         for (int w = 0; w < NW; ++w) v += part[w * NE * 64 * 4 + idx];
-        if (B) v += to_f32(B[n]);
-        Y[(t0 + t) * N + n] = from_f32<T>(v);
+        if (B) v += to_f32(B[n0 + n]);
+        Y[(t0 + t) * N + n0 + n] = from_f32<T>(v);
     }
 }
 
@@ -149,7 +150,8 @@ int linear_skinny_mfma(const void *X, const void *W, const void *B, int64_t Ttok
     T *y = static_cast<T *>(Y);
     if (N <= 16) linear_skinny_mfma_kernel<T, 1, NW><<<grid, NW * 64, 0, s>>>(x, w, b, Ttok, K, N, y);
     else if (N <= 32) linear_skinny_mfma_kernel<T, 2, NW><<<grid, NW * 64, 0, s>>>(x, w, b, Ttok, K, N, y);
-    else linear_skinny_mfma_kernel<T, 4, NW><<<grid, NW * 64, 0, s>>>(x, w, b, Ttok, K, N, y);
+    else   // 64 outputs per block; more outputs: more blocks over the same tokens (X read once per 64 outputs)
+        linear_skinny_mfma_kernel<T, 4, NW><<<dim3(grid, static_cast<unsigned>(ceil_div(N, 64))), NW * 64, 0, s>>>(x, w, b, Ttok, K, N, y);
     OPMX_LAUNCH_CHECK();
     return OPMX_OK;
 }
@@ -190,9 +192,11 @@ int launch_linear(const void *X, const void *W, const void *B, int64_t T, int64_
     // Few outputs, many tokens: the MFMA kernel that splits K over the waves of a block.  Measured
     // against the other two (H = 4096, 8 outputs: 10 us against 19 at T = 4096, 18 against 30 at
     // 8192, no gain below; H = 2048, 64 outputs: 12-13 us against the tile kernel's 21 from T = 512
-    // to 4096, while from 8192 tokens on the tile kernel re-reads W less and wins).
-    if ((dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16) && N <= 64 && K >= 32 && K % 32 == 0 && aligned16(X) &&
-        aligned16(W) && (N <= 8 ? T >= 4096 : (T >= 512 && (N <= 16 || T < 8192))))
+    // to 4096, while from 8192 tokens on the tile kernel re-reads W less and wins; H = 7168, 256 outputs
+    // in four blocks of 64 over the same tokens: 37 us against 64 up to T = 1024, 71 against 64 at 2048).
+    if ((dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16) && N <= 256 && K >= 32 && K % 32 == 0 && aligned16(X) &&
+        aligned16(W) &&
+        (N <= 8 ? T >= 4096 : N <= 64 ? (T >= 512 && (N <= 16 || T < 8192)) : (T >= 512 && T * N <= 262144)))
         return dtype == OPMX_DTYPE_F16 ? linear_skinny_mfma<f16>(X, W, B, T, K, N, Y, s)
                                        : linear_skinny_mfma<bf16>(X, W, B, T, K, N, Y, s);
     if ((dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16) && T >= 512 && N > 8 && K % 64 == 0 &&
