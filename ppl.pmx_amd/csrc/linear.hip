@@ -193,10 +193,12 @@ int launch_linear(const void *X, const void *W, const void *B, int64_t T, int64_
     // against the other two (H = 4096, 8 outputs: 10 us against 19 at T = 4096, 18 against 30 at
     // 8192, no gain below; H = 2048, 64 outputs: 12-13 us against the tile kernel's 21 from T = 512
     // to 4096, while from 8192 tokens on the tile kernel re-reads W less and wins; H = 7168, 256 outputs
-    // in four blocks of 64 over the same tokens: 37 us against 64 up to T = 1024, 71 against 64 at 2048).
+    // in four blocks of 64 over the same tokens: 37 us against 64 up to T = 1024, 71 against 64 at 2048;
+    // its K chain costs about H / 195 us whatever T is, which one block per token undercuts up to
+    // T * N of about 32768: 256 outputs, T = 128: 31 us per-token blocks, 36 us this kernel; T = 256: 61 / 37).
     if ((dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16) && N <= 256 && K >= 32 && K % 32 == 0 && aligned16(X) &&
         aligned16(W) &&
-        (N <= 8 ? T >= 4096 : N <= 64 ? (T >= 512 && (N <= 16 || T < 8192)) : (T >= 512 && T * N <= 262144)))
+        (N <= 8 ? T >= 4096 : N <= 64 ? (T >= 512 && (N <= 16 || T < 8192)) : (T * N >= 32768 && T * N <= 262144)))
         return dtype == OPMX_DTYPE_F16 ? linear_skinny_mfma<f16>(X, W, B, T, K, N, Y, s)
                                        : linear_skinny_mfma<bf16>(X, W, B, T, K, N, Y, s);
     if ((dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16) && T >= 512 && N > 8 && K % 64 == 0 &&

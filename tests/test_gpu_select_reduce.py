@@ -190,6 +190,7 @@ def test_swiglu_and_silu(R, D, dtype):
                                               (8192, 2048, 64, torch.bfloat16, True),   # back on the tile kernel
                                               (1000, 1024, 256, torch.bfloat16, True),  # 256 outputs: four blocks of 64 per token tile
                                               (600, 512, 100, torch.float16, False),    # last block of outputs ragged
+                                              (130, 256, 256, torch.bfloat16, True),    # 256 outputs from 128 tokens on
                                               (3000, 512, 200, torch.float16, True)])   # too many tokens for that: tile kernel
 def test_router_linear(T, K, N, dtype, bias):
     g = torch.Generator().manual_seed(K + N)
