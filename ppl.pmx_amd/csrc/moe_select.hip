@@ -54,7 +54,10 @@ __device__ __forceinline__ void route_token(const T *srow, int E, int k, int G, 
     }
     my_id = -1;
     float my_v = 0.0f;
-    if (G == kWave) {
+    // With several keys per lane (E > 64) the ranking below costs E broadcasts of up to four
+    // compares each; the k rounds of the other branch are cheaper there (E = 256, k = 8: MoeSelect at
+    // T = 512 51 -> 38 us, at T = 8192 291 -> 247 us), so only one key per lane is ranked.
+    if (G == kWave && vpl == 1) {
         // A whole wave routes the token.  Keys are distinct (the id is part of the key),
         // so "how many keys beat mine" is the key's position in the descending order:
         // E scalar broadcasts and compares, no k-round dependency chain.  The key of
