@@ -29,7 +29,19 @@ __global__ __launch_bounds__(256) void moe_reduce_kernel(const T *__restrict__ Y
                 float acc[n];
 #pragma unroll
                 for (int i = 0; i < n; ++i) acc[i] = 0.0f;
-                for (int s = 0; s < k; ++s) {
+                int s = 0;
+                for (; s + 4 <= k; s += 4) {       // four gathered rows in flight; summed in slot order
+                    Vec16<T> v[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) v[u] = load16(Y + srow[s + u] * N + c);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const float ws = sw[s + u];
+#pragma unroll
+                        for (int i = 0; i < n; ++i) acc[i] += ws * to_f32(v[u].v[i]);
+                    }
+                }
+                for (; s < k; ++s) {
                     Vec16<T> v = load16(Y + srow[s] * N + c);
                     float ws = sw[s];
 #pragma unroll
