@@ -88,6 +88,23 @@ int opmx_moe_select(const void *X, const void *scores, int64_t T, int64_t H, int
                     int64_t *invert_permutation, int64_t *expert_offset, int32_t *expert_ids,
                     void *workspace, size_t workspace_bytes, void *stream);
 
+/* MoeSelect for callers that cannot allocate device memory (code under HIP graph capture,
+ * serving loops and harnesses that forbid hipMalloc).  No counterpart in the reference: it is
+ * opmx_moe_select without the workspace argument, with the same inputs, outputs, limits and
+ * results.  The scratch memory (chunk histograms and picked ids of calls with more than 256
+ * tokens) is an array of OPMX_MOE_SELECT_STATIC_SCRATCH_BYTES bytes inside the library that
+ * every GPU the library runs on holds until the process ends; the call allocates and frees
+ * nothing.  A call whose opmx_moe_select_workspace_bytes(T, E, k) exceeds that size returns
+ * OPMX_ERR_WORKSPACE (nothing enqueued).  All calls on one GPU share the array: two calls
+ * that overlap on one GPU (different streams or threads) race; calls ordered on one stream
+ * do not.  The first call on a GPU looks the array's address up and must be outside a
+ * stream capture. */
+#define OPMX_MOE_SELECT_STATIC_SCRATCH_BYTES (4u << 20)
+int opmx_moe_select_static(const void *X, const void *scores, int64_t T, int64_t H, int E, int k,
+                           int dtype, void *X_expand_permute, void *expert_weights,
+                           int64_t *invert_permutation, int64_t *expert_offset, int32_t *expert_ids,
+                           void *stream);
+
 /* Router gate and MoeSelect in one call: scores = X gate_weight^T (+ gate_bias), then
  * opmx_moe_select on those scores.  Replaces the pair of calls at
  * model_zoo/mixtral/modeling/dynamic_batching/Model.py:188-190 (self.gate, then

@@ -145,6 +145,23 @@ int opmx_moe_select(const void *X, const void *scores, int64_t T, int64_t H, int
                              expert_offset, expert_ids, workspace, st(stream));
 }
 
+int opmx_moe_select_static(const void *X, const void *scores, int64_t T, int64_t H, int E, int k, int dtype,
+                           void *X_expand_permute, void *expert_weights, int64_t *invert_permutation,
+                           int64_t *expert_offset, int32_t *expert_ids, void *stream)
+{
+    if (T < 0 || H < 0 || E <= 0 || k <= 0 || k > E) return OPMX_ERR_BAD_ARGUMENT;
+    if (!dtype_ok(dtype) || E > OPMX_MOE_MAX_EXPERTS || k > OPMX_MOE_MAX_EXPERTS_PER_TOKEN)
+        return OPMX_ERR_UNSUPPORTED;
+    if (T > (int64_t{1} << 31) / k) return OPMX_ERR_UNSUPPORTED;
+    if (!expert_offset) return OPMX_ERR_BAD_ARGUMENT;
+    if (T > 0 && (!scores || !expert_weights || !invert_permutation)) return OPMX_ERR_BAD_ARGUMENT;
+    if (T > 0 && H > 0 && (!X || !X_expand_permute)) return OPMX_ERR_BAD_ARGUMENT;
+    // more tokens than the library's own scratch memory holds: rejected on the host
+    if (moe_select_workspace_bytes(T, E, k) > OPMX_MOE_SELECT_STATIC_SCRATCH_BYTES) return OPMX_ERR_WORKSPACE;
+    return launch_moe_select_static(X, scores, T, H, E, k, dtype, X_expand_permute, expert_weights,
+                                    invert_permutation, expert_offset, expert_ids, st(stream));
+}
+
 int opmx_moe_route_select(const void *X, const void *gate_weight, const void *gate_bias, int64_t T, int64_t H, int E,
                           int k, int dtype, void *scores, void *X_expand_permute, void *expert_weights,
                           int64_t *invert_permutation, int64_t *expert_offset, int32_t *expert_ids, void *workspace,

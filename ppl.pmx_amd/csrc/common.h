@@ -80,6 +80,8 @@ int launch_moe_select(const void *X, const void *scores, int64_t T, int64_t H, i
                       void *Xp, void *w, int64_t *inv, int64_t *off, int32_t *ids, void *ws,
                       hipStream_t s);
 size_t moe_select_workspace_bytes(int64_t T, int E, int k);
+int launch_moe_select_static(const void *X, const void *scores, int64_t T, int64_t H, int E, int k, int dtype,
+                             void *Xp, void *w, int64_t *inv, int64_t *off, int32_t *ids, hipStream_t s);
 int launch_moe_route_select(const void *X, const void *Wg, const void *Bg, int64_t T, int64_t H, int E, int k,
                             int dtype, void *scores, void *Xp, void *w, int64_t *inv, int64_t *off, int32_t *ids,
                             void *ws, hipStream_t s);

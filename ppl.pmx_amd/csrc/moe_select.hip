@@ -6,6 +6,8 @@
 //   expert_offset[e] + (#tokens before it that picked e)
 // and the count is taken from bit matrices (one bit per (expert, token)), whose
 // construction by atomicOr is order independent.
+#include <mutex>
+
 #include "moe_gemm.h"
 
 namespace opmx {
@@ -559,6 +561,49 @@ int launch_moe_select(const void *X, const void *scores, int64_t T, int64_t H, i
         case OPMX_DTYPE_BF16: return select_impl<bf16>(X, scores, T, H, E, k, Xp, w, inv, off, ids, ws, s);
     }
     return OPMX_ERR_UNSUPPORTED;
+}
+
+// ---- MoeSelect for callers that cannot allocate ----
+// The chunk histograms and the picked ids of the many-token path live in this array instead of a
+// caller's workspace.  Each GPU holds its own copy at its own address; host code never uses the
+// array's name as an address, only the pointer hipGetSymbolAddress returned for that GPU.
+static __device__ __align__(256) unsigned char scratch[OPMX_MOE_SELECT_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+void *scratch_ptr[kMaxDevices];   // by device ordinal; written under scratch_mutex
+
+// The address of `scratch` on the GPU that is current on this thread (looked up once per GPU).
+int scratch_for_current_device(void **out)
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return OPMX_ERR_LAUNCH;
+    std::lock_guard<std::mutex> hold(scratch_mutex);
+    if (scratch_ptr[dev] == nullptr) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) {
+            (void)hipGetLastError();
+            return OPMX_ERR_LAUNCH;
+        }
+        scratch_ptr[dev] = p;
+    }
+    *out = scratch_ptr[dev];
+    return OPMX_OK;
+}
+}  // namespace
+
+// Every kernel of select_impl writes the part of the scratch memory it later reads (all chunk
+// histograms of the call, all picked ids), so nothing has to start at zero and what the
+// previous call left behind is never read.
+int launch_moe_select_static(const void *X, const void *scores, int64_t T, int64_t H, int E, int k, int dtype,
+                             void *Xp, void *w, int64_t *inv, int64_t *off, int32_t *ids, hipStream_t s)
+{
+    if (moe_select_workspace_bytes(T, E, k) > sizeof(scratch)) return OPMX_ERR_WORKSPACE;
+    void *ws = nullptr;
+    const int rc = scratch_for_current_device(&ws);
+    if (rc != OPMX_OK) return rc;
+    return launch_moe_select(X, scores, T, H, E, k, dtype, Xp, w, inv, off, ids, ws, s);
 }
 
 }  // namespace opmx

@@ -20,6 +20,7 @@ ABI_VERSION = 1
 F32, F16, BF16 = 0, 1, 2
 EPILOGUE_NONE, EPILOGUE_SWIGLU = 0, 1
 MAX_EXPERTS, MAX_EXPERTS_PER_TOKEN = 256, 32
+SELECT_STATIC_SCRATCH_BYTES = 4 << 20
 
 _DTYPES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 _lib = None
@@ -31,6 +32,7 @@ _SIGNATURES = {
     "opmx_linear": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp, _vp]),
     "opmx_moe_select_workspace_bytes": (_sz, [_i64, _int, _int]),
     "opmx_moe_select": (_int, [_vp, _vp, _i64, _i64, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "opmx_moe_select_static": (_int, [_vp, _vp, _i64, _i64, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp]),
     "opmx_moe_route_select": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                      _sz, _vp]),
     "opmx_moe_grouped_gemm_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _int]),

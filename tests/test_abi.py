@@ -54,6 +54,17 @@ def test_argument_validation_needs_no_device(lib):
     assert lib.opmx_moe_select(one, one, 4, 8, 8, 2, 1, one, one, one, one, None, None, 0, None) == -3      # workspace
     assert lib.opmx_moe_select(one, one, 4, 8, 8, 2, 1, one, one, one, one, None, P(8), 1 << 20, None) == -4  # align
     assert lib.opmx_moe_select(None, one, 4, 8, 8, 2, 1, one, one, one, one, None, one, 1 << 20, None) == -1
+    # the variant with the library's own scratch array: same checks, and sizes beyond the array
+    from torch_function import _lib
+    st = lambda *a: lib.opmx_moe_select_static(*a)
+    assert st(one, one, 4, 8, 8, 9, 1, one, one, one, one, None, None) == -1    # k > E
+    assert st(one, one, 4, 8, 300, 2, 1, one, one, one, one, None, None) == -2  # E
+    assert st(one, one, 4, 8, 8, 2, 7, one, one, one, one, None, None) == -2    # dtype
+    assert st(None, one, 4, 8, 8, 2, 1, one, one, one, one, None, None) == -1
+    assert lib.opmx_moe_select_workspace_bytes(1 << 20, 8, 2) > _lib.SELECT_STATIC_SCRATCH_BYTES
+    assert st(one, one, 1 << 20, 64, 8, 2, 1, one, one, one, one, None, None) == -3   # 8 MB of ids alone
+    assert lib.opmx_moe_select_workspace_bytes(1 << 18, 64, 8) > _lib.SELECT_STATIC_SCRATCH_BYTES
+    assert st(one, one, 1 << 18, 64, 64, 8, 2, one, one, one, one, None, None) == -3
     # router gate + select in one call: the argument checks of opmx_moe_select
     rs = lambda *a: lib.opmx_moe_route_select(*a)
     assert rs(one, one, None, 4, 8, 8, 9, 1, one, one, one, one, one, None, one, 1 << 20, None) == -1   # k > E
