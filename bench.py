@@ -6,7 +6,12 @@ MoeSelect -> gate/up grouped GEMM -> SwiGLU -> down grouped GEMM -> MoeReduce)
 through the drop-in operators, over one batch of synthetic tokens that is
 already resident in HBM.  Prints ONE JSON line:
 
-  value / ms_per_step  whole-layer tokens/s and latency over exactly --steps steps
+  value / ms_per_step  whole-layer tokens/s and latency over exactly --steps steps (the first timed
+                       window, after --warmup untimed steps)
+  conditioning         untimed layer steps run before the warm-up (--conditioning-ms of them): a
+                       device that has been idle takes some ten milliseconds of work to reach its
+                       sustained clocks, more than a short --warmup covers
+  windows              ms/step of further windows of --steps steps each (min / median / max)
   roofline             the dominant kernel (gate/up grouped GEMM): algorithmic bytes
                        or flops per launch / mean launch duration (HIP events on
                        the launch stream, taken inside the timed steps) vs MI355X peak
@@ -19,8 +24,16 @@ already resident in HBM.  Prints ONE JSON line:
   vendor_dense_gemm_same_flops_TFLOPs
                        MFMA-bound workloads: the vendor library's dense GEMM with the flop
                        count of the gate/up launch (no expert grouping), context only
+  companion            with the default workload: every other configuration of the benchmark set
+                       (decode T=1/8/128, T=512/1024, prefill T=2048/8192, 64 experts T=32/4096,
+                       8x22B shape T=16/4096), each measured by a child process of this program
   cpu_baseline         the CPU oracle (PyTorch CPU restatement of the reference
                        operator sequence) on the host cores, bounded sample
+
+Inputs: x ~ N(0,1) and the router weight ~ N(0,0.02) are drawn on the CPU under
+torch.manual_seed(0), x first, so the routing (expert shares, active experts) is that of the seeded
+tensor set; the expert weights ~ N(0,0.02), whose values influence neither routing nor timing, are
+drawn on the device unless --cpu-weights asks for the CPU draws as well (about a minute).
 
 Workloads (--workload): decode-T{1,8,32,128} and prefill-T{2048,8192} at the
 Mixtral-8x7B shape (fp16), fine-T{32,4096} (64 experts, top-8, bf16),
@@ -41,14 +54,47 @@ for p in (ROOT, os.path.join(ROOT, "ppl.pmx_amd")):
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, vendor figure
 MFMA_PEAK_TFLOPS = 2500.0      # dense fp16/bf16 MFMA, vendor figure
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this program, each scaled by the same counter's reading for a plain copy kernel of known size
-# (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000): profiles/gemm_stream_decode_T32_mixtral8x7b.txt and
-# profiles/gemm_tiled_prefill_T8192_mixtral8x7b.txt.  None where no counter run was made.
-MEASURED_TRAFFIC = {
-    ("decode-T32", False): 1883394048 + 3674624,
-    ("prefill-T8192", False): 2 * 3859194 * 1024 + 917504 * 1024,
-}
+# HBM bytes per launch of the dominant kernel come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# of this program, each scaled by the same counter's reading for a plain copy kernel of known size.
+# The summaries under profiles/ record them in a line
+#   bench-traffic: workload=<name> fused_swiglu=<0|1> bytes_per_launch=<n> kernel_sources_sha256=<hex>
+# together with the hash of the kernel sources the counter run was made with; a line whose hash
+# is not that of the sources in this tree is out of date and is not reported.
+def kernel_sources_sha256():
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "ppl.pmx_amd", "csrc")
+    for path in sorted(glob.glob(os.path.join(csrc, "*.hip")) + glob.glob(os.path.join(csrc, "*.h"))):
+        if os.path.basename(path) == "device_ceilings.hip":
+            continue
+        h.update(os.path.basename(path).encode())
+        h.update(open(path, "rb").read())
+    return h.hexdigest()
+
+
+def measured_traffic(workload, fused):
+    """(bytes per launch or None, where the figure comes from / why there is none)."""
+    import glob
+    import re
+    want = kernel_sources_sha256()
+    stale = None
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.txt"))):
+        for m in re.finditer(r"bench-traffic: workload=(\S+) fused_swiglu=([01]) bytes_per_launch=(\d+) "
+                             r"kernel_sources_sha256=([0-9a-f]+)", open(path).read()):
+            if m.group(1) != workload or bool(int(m.group(2))) != bool(fused):
+                continue
+            rel = os.path.relpath(path, ROOT)
+            if m.group(4) == want:
+                return int(m.group(3)), rel
+            stale = "{}: counter run made with other kernel sources, not reported".format(rel)
+    return None, stale or "no counter run for this workload under profiles/"
+
+
+# configurations of the benchmark set measured beside the default workload (child processes)
+COMPANIONS = [("decode-T1", []), ("decode-T8", []), ("decode-T128", []), ("decode-T512", []), ("decode-T1024", []),
+              ("prefill-T2048", []), ("prefill-T8192", []), ("prefill-T8192", ["--fuse-swiglu"]),
+              ("fine-T32", []), ("fine-T4096", []), ("8x22b-T16", []), ("8x22b-T4096", [])]
 
 SHAPES = {
     "decode": dict(H=4096, E=8, k=2, I=14336, dtype="float16", skew=0.0, name="mixtral-8x7b"),
@@ -77,6 +123,11 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="decode-T32")
+    ap.add_argument("--conditioning-ms", type=float, default=300.0,
+                    help="untimed layer steps for this long before the warm-up (reported, never timed)")
+    ap.add_argument("--windows", type=int, default=4, help="further timed windows of --steps steps (min/median/max)")
+    ap.add_argument("--cpu-weights", action="store_true",
+                    help="draw the expert weights on the CPU too, after x and the router weight (slow)")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay leg")
     ap.add_argument("--event-stride", type=int, default=8,
                     help="HIP events around every n-th launch of the dominant kernel inside the timed steps")
@@ -94,7 +145,12 @@ def main():
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
                     help="also run N plain device-to-device copies of the gate/up weight tensor (known size): "
                          "the reference reading for FETCH_SIZE / WRITE_SIZE counter runs")
+    ap.add_argument("--kernel-sources-hash", action="store_true",
+                    help="print the hash that a bench-traffic line under profiles/ must carry for this tree, and exit")
     args = ap.parse_args()
+    if args.kernel_sources_hash:
+        print(kernel_sources_sha256())
+        return
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (TP=1, no collectives); --gpus {} is not "
                  "supported, run with --gpus 1".format(args.gpus))
@@ -114,23 +170,24 @@ def main():
                                                  check=True).stdout.strip().splitlines()[-1])
         except Exception as exc:   # the probe is optional
             print("device ceiling probe failed: {}".format(exc), file=sys.stderr)
-    # The default run (decode, HBM-bound) also reports the MFMA-bound companion workload of the
-    # same layer, prefill T=8192 with skewed routing, as six operators and with the SwiGLU
-    # epilogue: child processes of this program, run while this one leaves the GPU idle.
+    # The default run also measures every other configuration of the benchmark set: child
+    # processes of this program, run one after the other while this one leaves the GPU idle.
     companion = None
     if args.workload == "decode-T32" and not args.no_companion:
         import subprocess
         companion = {}
-        for name, extra in (("prefill-T8192", []), ("prefill-T8192, fused SwiGLU epilogue", ["--fuse-swiglu"])):
-            cmd = [sys.executable, os.path.abspath(__file__), "--workload", "prefill-T8192", "--steps", "50", "--warmup", "5",
-                   "--no-cpu-baseline", "--no-device-ceilings", "--no-vendor-gemm", "--no-companion"] + extra
+        for name, extra in COMPANIONS:
+            cmd = [sys.executable, os.path.abspath(__file__), "--workload", name, "--steps", "50", "--warmup", "5",
+                   "--windows", "2", "--no-cpu-baseline", "--no-device-ceilings", "--no-vendor-gemm",
+                   "--no-companion"] + extra
             try:
                 line = subprocess.run(cmd, capture_output=True, text=True, timeout=300, check=True).stdout.strip().splitlines()[-1]
                 r = json.loads(line)
-                companion[name] = {key: r[key] for key in ("value", "unit", "ms_per_step", "steps", "config", "roofline",
-                                                           "layer", "hip_graph_replay", "per_op_us")}
+                companion[name + (", fused SwiGLU epilogue" if extra else "")] = {
+                    key: r[key] for key in ("value", "unit", "ms_per_step", "steps", "windows", "config", "roofline",
+                                            "layer", "hip_graph_replay", "per_op_us")}
             except Exception as exc:
-                print("companion workload failed: {}".format(exc), file=sys.stderr)
+                print("companion workload {} failed: {}".format(name, exc), file=sys.stderr)
 
     import torch_function as OPMX
     from model_zoo.mixtral.modeling.dynamic_batching.Model import MoeFeedForward
@@ -142,15 +199,23 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
-    # ---- synthetic inputs, seeded, drawn on the device (x~N(0,1), weights~N(0,0.02))
-    g = torch.Generator(device="cuda").manual_seed(0)
-    x = torch.randn(T, H, generator=g, device=dev).to(dtype)
+    # ---- synthetic inputs: x and the router weight from the CPU generator under seed 0 (x first),
+    # so the routing is that of the seeded tensor set; expert weights on the device (see above)
+    gc = torch.Generator().manual_seed(0)
+    x = torch.randn(T, H, generator=gc).to(dtype).to(dev)
     layer = MoeFeedForward(MoeFeedForward.params(H, I, E, k), 0, True, False, None, dtype=dtype, device=dev,
                            fuse_swiglu_epilogue=args.fuse_swiglu)
-    layer.gate.weight.data = (torch.randn(E, H, generator=g, device=dev) * 0.02).to(dtype)
-    for e in range(E):
-        layer.wu.weight.data[e] = (torch.randn(2 * I, H, generator=g, device=dev) * 0.02).to(dtype)
-        layer.w2.weight.data[e] = (torch.randn(H, I, generator=g, device=dev) * 0.02).to(dtype)
+    layer.gate.weight.data = (torch.randn(E, H, generator=gc) * 0.02).to(dtype).to(dev)
+    g = torch.Generator(device="cuda").manual_seed(0)
+    if args.cpu_weights:
+        for e in range(E):
+            layer.wu.weight.data[e] = (torch.randn(2 * I, H, generator=gc) * 0.02).to(dtype).to(dev)
+        for e in range(E):
+            layer.w2.weight.data[e] = (torch.randn(H, I, generator=gc) * 0.02).to(dtype).to(dev)
+    else:
+        for e in range(E):
+            layer.wu.weight.data[e] = (torch.randn(2 * I, H, generator=g, device=dev) * 0.02).to(dtype)
+            layer.w2.weight.data[e] = (torch.randn(H, I, generator=g, device=dev) * 0.02).to(dtype)
     if cfg["skew"] > 0:       # Zipf(s=1.2) per-expert logit bias: skewed expert load
         p = torch.arange(1, E + 1, dtype=torch.float64) ** -1.2
         bias = (cfg["skew"] * torch.log(p / p.sum())).to(dtype).to(dev)
@@ -182,9 +247,37 @@ def main():
         out = timed("moe_reduce", lambda: OPMX.moe_reduce(y, w, inv, k))
         return out, off
 
+    def step(i=-1, ev=None, stride=1):
+        if args.fuse_router_select:
+            xe, w, inv, off, sc = OPMX.moe_route_select(x, Wg, gb, E, k)
+        else:
+            sc = OPMX.linear(x, Wg, gb, H, E)
+            xe, w, inv, off = OPMX.moe_select(x, sc, E, k)
+        mark = ev is not None and i % stride == 0
+        if mark:
+            ev[i // stride][0].record()
+        h = gemm1(xe, off)
+        if mark:
+            ev[i // stride][1].record()
+        act = h if args.fuse_swiglu else OPMX.swiglu(h)
+        y = OPMX.moe_row_parallel_linear(act, off, w2, None, None, E, I, H, True)
+        return OPMX.moe_reduce(y, w, inv, k)
+
+    def window(n, ev=None, stride=1):
+        """n steps between two device synchronisations -> ms per step"""
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(n):
+            step(i, ev, stride)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n * 1e3
+
+    gemm1 = (lambda xe, off: OPMX.moe_column_parallel_linear_swiglu(xe, off, wu, None, E, H, 2 * I)) \
+        if args.fuse_swiglu else \
+        (lambda xe, off: OPMX.moe_column_parallel_linear(xe, off, wu, None, None, E, H, 2 * I, False))
+
     with torch.inference_mode():
-        for _ in range(max(args.warmup, 1)):
-            out, off = ops()
+        out, off = ops()
         torch.cuda.synchronize()
         counts = (off[1:] - off[:-1]).cpu()
         active = int((counts > 0).sum())
@@ -192,35 +285,35 @@ def main():
         if cfg["kind"] == "prefill":
             assert float(counts.max()) / R > 0.40, "skewed-routing config needs the largest expert above 40%"
 
-        # ---- timed region: exactly --steps steps; HIP events bracket the dominant kernel
-        # events around every `stride`-th launch of the dominant kernel (at least 8 of them): an event
-        # record is a barrier packet in the queue, and two per step cost the eager steps 1-3 %
+        # ---- conditioning (untimed, reported): layer steps until the device has been busy for
+        # --conditioning-ms.  Straight out of idle the same kernels run 8-10 % slower for the first
+        # ten milliseconds or so, which a warm-up of a few steps does not cover.
+        cond_steps, c0 = 0, time.perf_counter()
+        while (time.perf_counter() - c0) * 1e3 < args.conditioning_ms:
+            for _ in range(8):
+                step()
+            cond_steps += 8
+            torch.cuda.synchronize()
+        cond_ms = (time.perf_counter() - c0) * 1e3
+
+        # ---- warm-up, then the timed region: exactly --steps steps; HIP events bracket the dominant
+        # kernel at every `stride`-th launch (at least 8 of them): an event record is a barrier
+        # packet in the queue, and two per step cost the eager steps 1-3 %
+        for _ in range(args.warmup):
+            step()
         stride = max(1, min(args.event_stride, args.steps // 8 if args.steps >= 8 else 1))
         ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
               for _ in range((args.steps + stride - 1) // stride)]
-        gemm1 = (lambda xe, off: OPMX.moe_column_parallel_linear_swiglu(xe, off, wu, None, E, H, 2 * I)) \
-            if args.fuse_swiglu else \
-            (lambda xe, off: OPMX.moe_column_parallel_linear(xe, off, wu, None, None, E, H, 2 * I, False))
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(args.steps):
-            if args.fuse_router_select:
-                xe, w, inv, off, sc = OPMX.moe_route_select(x, Wg, gb, E, k)
-            else:
-                sc = OPMX.linear(x, Wg, gb, H, E)
-                xe, w, inv, off = OPMX.moe_select(x, sc, E, k)
-            if i % stride == 0:
-                ev[i // stride][0].record()
-            h = gemm1(xe, off)
-            if i % stride == 0:
-                ev[i // stride][1].record()
-            act = h if args.fuse_swiglu else OPMX.swiglu(h)
-            y = OPMX.moe_row_parallel_linear(act, off, w2, None, None, E, I, H, True)
-            out = OPMX.moe_reduce(y, w, inv, k)
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-        ms_per_step = dt / args.steps * 1e3
+        ms_per_step = window(args.steps, ev, stride)
         gemm1_ms = sum(a.elapsed_time(b) for a, b in ev) / len(ev)
+        # further windows of the same length, for the spread
+        more = sorted(window(args.steps) for _ in range(max(args.windows, 0)))
+        windows = None
+        if more:
+            windows = {"n": len(more), "steps_each": args.steps, "ms_per_step_min": round(more[0], 4),
+                       "ms_per_step_median": round(more[len(more) // 2] if len(more) % 2 else
+                                                   0.5 * (more[len(more) // 2 - 1] + more[len(more) // 2]), 4),
+                       "ms_per_step_max": round(more[-1], 4)}
 
         # ---- the same steps replayed from a captured HIP graph: what a serving loop does when the
         # host's launch path (six operators per layer) is slower than the GPU work, i.e. at few
@@ -232,7 +325,12 @@ def main():
                 cg = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(cg):
                     ops()
-                for _ in range(max(args.warmup, 1)):
+                c0 = time.perf_counter()
+                while (time.perf_counter() - c0) * 1e3 < args.conditioning_ms / 3:
+                    for _ in range(8):
+                        cg.replay()
+                    torch.cuda.synchronize()
+                for _ in range(args.warmup):
                     cg.replay()
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
@@ -288,12 +386,13 @@ def main():
     gemm1_flops = 2.0 * R * H * 2 * I
     layer_bytes = w_bytes_gemm1 + w_bytes_gemm2 + 2 * T * H * s + E * H * s
     layer_flops = T * (k * (2.0 * H * 2 * I + 2.0 * I * H) + 2.0 * H * E)
+    traffic, traffic_source = measured_traffic(args.workload, args.fuse_swiglu)
     hbm_bound = (layer_flops / layer_bytes) < (MFMA_PEAK_TFLOPS * 1e12) / (HBM_PEAK_GBS * 1e9)
     if hbm_bound:
         ach = gemm1_bytes / (gemm1_ms * 1e-3) / 1e9
         roof = dict(bound="hbm", kernel="gate_up_grouped_gemm", achieved=round(ach, 1), peak=HBM_PEAK_GBS,
                     unit="GB/s", frac=round(ach / HBM_PEAK_GBS, 4),
-                    traffic=MEASURED_TRAFFIC.get((args.workload, args.fuse_swiglu)),
+                    traffic=traffic, traffic_source=traffic_source,
                     algorithmic_bytes=int(gemm1_bytes), launch_ms=round(gemm1_ms, 4))
         lach = layer_bytes / (ms_per_step * 1e-3) / 1e9
         lay = dict(bound="hbm", achieved=round(lach, 1), peak=HBM_PEAK_GBS, unit="GB/s",
@@ -302,7 +401,7 @@ def main():
         ach = gemm1_flops / (gemm1_ms * 1e-3) / 1e12
         roof = dict(bound="mfma", kernel="gate_up_grouped_gemm", achieved=round(ach, 1), peak=MFMA_PEAK_TFLOPS,
                     unit="TFLOP/s", frac=round(ach / MFMA_PEAK_TFLOPS, 4),
-                    traffic=MEASURED_TRAFFIC.get((args.workload, args.fuse_swiglu)),
+                    traffic=traffic, traffic_source=traffic_source,
                     algorithmic_flops=int(gemm1_flops), launch_ms=round(gemm1_ms, 4))
         lach = layer_flops / (ms_per_step * 1e-3) / 1e12
         lay = dict(bound="mfma", achieved=round(lach, 1), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
@@ -319,6 +418,7 @@ def main():
         "metric": "MoE-layer tokens/sec at Mixtral-8x7B shape, fp16, 1 GPU; % HBM/MFMA roofline",
         "value": round(T / (ms_per_step * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "conditioning": {"steps": cond_steps, "ms": round(cond_ms, 1), "timed": False}, "windows": windows,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {"float16": "f16", "bfloat16": "bf16"}[cfg["dtype"]], "data": "synthetic",
         "config": {"workload": "{} MoE layer {}, T={} tokens, hidden={}, experts={}, top-{}, ffn={}, TP=1".format(

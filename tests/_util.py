@@ -9,20 +9,22 @@ def dev():
 
 
 def gpu_inputs(T, H, E, I, dtype, seed=0):
-    """Seeded x, Wg, wu, w2 drawn on the GPU (large configs would take minutes on
-    the host) and returned as (device tensors, host copies): both paths under
-    test see identical bits."""
-    g = torch.Generator(device="cuda").manual_seed(seed)
+    """Seeded x, Wg, wu, w2, returned as (device tensors, host copies): both paths under test see
+    identical bits.  x and the router weight are the CPU draws of the oracle's `make_inputs`
+    (x first), so the routing is that of the seeded tensor set; the expert weights, which would
+    take minutes to draw on the host at the large configurations, are drawn on the GPU."""
+    from oracle import moe_oracle as O
     d = dev()
-    x = torch.randn(T, H, generator=g, device=d).to(dtype)
-    Wg = (torch.randn(E, H, generator=g, device=d) * 0.02).to(dtype)
+    xc, Wgc = O.make_inputs(T, H, E, I, dtype=dtype, seed=seed, with_w=False)
+    x, Wg = xc.to(d), Wgc.to(d)
+    g = torch.Generator(device="cuda").manual_seed(seed)
     wu = torch.empty(E, 2 * I, H, dtype=dtype, device=d)
     w2 = torch.empty(E, H, I, dtype=dtype, device=d)
     for e in range(E):
         wu[e] = (torch.randn(2 * I, H, generator=g, device=d) * 0.02).to(dtype)
         w2[e] = (torch.randn(H, I, generator=g, device=d) * 0.02).to(dtype)
     dev_t = (x, Wg, wu, w2)
-    return dev_t, tuple(t.cpu() for t in dev_t)
+    return dev_t, (xc, Wgc, wu.cpu(), w2.cpu())
 
 
 def assert_close_ulp(got, ref, dtype, ulps=2.0, what="", floor=1e-2):
