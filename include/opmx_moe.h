@@ -11,7 +11,16 @@
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
  *     all work is enqueued on it, nothing synchronises the device;
  *   - the library allocates nothing, frees nothing and keeps no pointer after
- *     a call returns; scratch memory comes in through `workspace`;
+ *     a call returns; scratch memory comes in through `workspace` (the one
+ *     exception, opmx_moe_select_static, says so below);
+ *   - process-wide state, all of it thread-safe: (1) the first launch of a kernel
+ *     on a GPU raises that kernel's shared-memory limit (hipFuncSetAttribute,
+ *     remembered per GPU and kernel) -- make one call per shape outside a stream
+ *     capture before capturing; (2) the compute-unit count of each GPU, looked up
+ *     once; (3) the tuning knobs of opmx_moe_set_option, whose initial values are
+ *     read once from the environment; (4) the per-GPU address of the scratch
+ *     array of opmx_moe_select_static.  Calls on different streams or threads do
+ *     not interfere as long as their buffers and workspaces differ;
  *   - every function returns OPMX_OK (0) or a negative opmx_status; on error
  *     nothing has been enqueued.  Faults inside a kernel surface, as with any
  *     HIP work, at the next synchronisation.
@@ -62,6 +71,21 @@ typedef enum opmx_epilogue {
 
 int opmx_moe_abi_version(void);
 const char *opmx_status_string(int status);
+
+/* Tuning / test knobs of the grouped GEMMs (no counterpart in the reference).  They choose
+ * between kernels that compute the same thing; results change at most in accumulation order.
+ * `name` is one of the strings below, `value` < 0 restores the automatic choice.  Each knob
+ * starts from the environment variable of the same name, read once when the library is first
+ * used (OPMX_MOE_GEMM accepts the words there).
+ *   "OPMX_MOE_GEMM"                1 generic, 2 tiled, 3 stream: force a kernel family
+ *   "OPMX_MOE_GEMM_TILED_VARIANT"  0 256x256 direct-to-LDS, 1 256x256 register-staged,
+ *                                  2 128x128 register-staged, 3 128x256 direct-to-LDS
+ *   "OPMX_MOE_GEMM_STREAM_VARIANT" 0..5: chunk widths / prefetch depth of the streaming kernel
+ *   "OPMX_MOE_GEMM_GNX"            tile order: 8 expert-major, 16 row partition, 4, 0 row-major
+ *   "OPMX_MOE_GEMM_STREAMK"        0 never split the tail tiles over K, 2 whenever possible
+ *   "OPMX_MOE_GEMM_PERSIST"        0 never the persistent form, 1 whenever its conditions hold
+ * Returns OPMX_ERR_BAD_ARGUMENT for an unknown name. */
+int opmx_moe_set_option(const char *name, int value);
 
 /* Router gate / plain linear.  Replaces Linear.forward,
  * torch_function/Linear.py:25-33 (called from

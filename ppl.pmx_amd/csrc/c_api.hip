@@ -1,6 +1,7 @@
 // extern "C" surface of libopmx_moe.so: argument checks and kernel selection.
 // Declarations and the reference operator each entry point replaces are in
 // include/opmx_moe.h.
+#include <atomic>
 #include <cstdlib>
 #include <cstring>
 
@@ -18,26 +19,58 @@ inline hipStream_t st(void *s) { return static_cast<hipStream_t>(s); }
 // at most 64 rows (measured crossover against the 128x256 MFMA tiles on MI355X).
 constexpr int64_t kStreamMaxRowsPerExpert = 64;
 
-int env_int(const char *name, int dflt)
+const char *const kOptionNames[kNumOptions] = {"OPMX_MOE_GEMM", "OPMX_MOE_GEMM_TILED_VARIANT",
+                                               "OPMX_MOE_GEMM_STREAM_VARIANT", "OPMX_MOE_GEMM_GNX",
+                                               "OPMX_MOE_GEMM_STREAMK", "OPMX_MOE_GEMM_PERSIST"};
+
+// Kernel family names accepted for OPMX_MOE_GEMM in the environment.
+int parse_option(int id, const char *v)
 {
-    const char *v = std::getenv(name);
-    return (v && *v) ? std::atoi(v) : dflt;
+    if (!v || !*v) return -1;
+    if (id == kOptGemm) {
+        if (!std::strcmp(v, "generic")) return 1;
+        if (!std::strcmp(v, "tiled")) return 2;
+        if (!std::strcmp(v, "stream")) return 3;
+    }
+    char *end = nullptr;
+    const long n = std::strtol(v, &end, 10);
+    return (end && *end == 0 && n >= 0 && n < 1000) ? static_cast<int>(n) : -1;
 }
 
-// 0 = automatic, 1 = generic, 2 = tiled, 3 = stream  (tuning / test knob)
-int forced_kernel()
+// The knobs: filled from the environment when first needed (thread-safe: initialisation of a
+// function-local static), changed afterwards only through opmx_moe_set_option.
+struct Options {
+    std::atomic<int> v[kNumOptions];
+    Options()
+    {
+        for (int i = 0; i < kNumOptions; ++i) v[i].store(parse_option(i, std::getenv(kOptionNames[i])));
+    }
+};
+Options &options()
 {
-    const char *v = std::getenv("OPMX_MOE_GEMM");
-    if (!v || !*v) return 0;
-    if (!std::strcmp(v, "generic")) return 1;
-    if (!std::strcmp(v, "tiled")) return 2;
-    if (!std::strcmp(v, "stream")) return 3;
-    return 0;
+    static Options o;
+    return o;
 }
+
+std::atomic<int> g_cu_count[kMaxDevices];
 
 }  // namespace
 
 namespace opmx {
+
+int option(Option o) { return options().v[o].load(std::memory_order_relaxed); }
+
+int cu_count()
+{
+    const int dev = current_device();
+    if (dev < 0) return 0;
+    int n = g_cu_count[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+        g_cu_count[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
 
 // Scratch memory that lets the 256x256 tile kernel balance its last rounds of tiles over all
 // CUs (stream-K); every kernel also runs without it.  256 bytes when the call would not use it.
@@ -68,7 +101,7 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
     const int64_t twice_mean = 2 * ceil_div(R, E);
     if (twice_mean < hint) hint = twice_mean;
     const bool stream_ws = true;   // the stream kernel needs no scratch memory
-    const int force = forced_kernel();
+    const int force = option(kOptGemm);      // 1 generic, 2 tiled, 3 stream, else automatic
 
     int choice;   // 1 generic, 2 tiled, 3 stream
     if (force == 3 && mfma_ok && stream_ws) choice = 3;
@@ -81,7 +114,7 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
 
     if (choice == 3)
         return launch_gemm_stream(X, off, W, B, E, R, K, N, dtype, epilogue, hint,
-                                  env_int("OPMX_MOE_GEMM_STREAM_VARIANT", 0), Y, s);
+                                  option(kOptStreamVariant) < 0 ? 0 : option(kOptStreamVariant), Y, s);
     if (choice == 2) {
         // The direct-to-LDS kernel takes 256x256 tiles unless they would fill the CUs less than
         // twice (the Mixtral down projection at T=2048: 1.3 rounds) or the experts hold fewer than
@@ -91,7 +124,7 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
         const int64_t tiles256 = (R / 256 + (E + 1) / 2) * ((out_cols + 255) / 256);
         const int dflt = R / E >= 128 && tiles256 >= 512 ? 0 : 3;
         return launch_gemm_tiled(X, off, W, B, E, R, K, N, dtype, epilogue,
-                                 env_int("OPMX_MOE_GEMM_TILED_VARIANT", dflt), Y, ws, ws_bytes, s);
+                                 option(kOptTiledVariant) < 0 ? dflt : option(kOptTiledVariant), Y, ws, ws_bytes, s);
     }
     return launch_gemm_generic(X, off, W, B, E, R, K, N, dtype, epilogue, Y, s);
 }
@@ -101,6 +134,17 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
 extern "C" {
 
 int opmx_moe_abi_version(void) { return OPMX_MOE_ABI_VERSION; }
+
+int opmx_moe_set_option(const char *name, int value)
+{
+    if (!name) return OPMX_ERR_BAD_ARGUMENT;
+    for (int i = 0; i < kNumOptions; ++i)
+        if (!std::strcmp(name, kOptionNames[i])) {
+            options().v[i].store(value < 0 ? -1 : value, std::memory_order_relaxed);
+            return OPMX_OK;
+        }
+    return OPMX_ERR_BAD_ARGUMENT;
+}
 
 const char *opmx_status_string(int status)
 {

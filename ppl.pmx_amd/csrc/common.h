@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "opmx_moe.h"
 
 namespace opmx {
@@ -67,6 +69,45 @@ __device__ __forceinline__ float sigmoid_fast_(float x)
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// ---- the little process-wide state the library keeps (all of it thread-safe) ----
+// Tuning / test knobs (opmx_moe_set_option; initial values from the environment variables of the
+// same names, read once).  -1 = automatic.  They select between kernels that compute the same
+// thing, never results beyond accumulation order.
+enum Option {
+    kOptGemm = 0,        // OPMX_MOE_GEMM: 1 generic, 2 tiled, 3 stream
+    kOptTiledVariant,    // OPMX_MOE_GEMM_TILED_VARIANT: 0..3
+    kOptStreamVariant,   // OPMX_MOE_GEMM_STREAM_VARIANT: 0..5
+    kOptGnx,             // OPMX_MOE_GEMM_GNX: tile order 0 / 4 / 8 / 16
+    kOptStreamK,         // OPMX_MOE_GEMM_STREAMK: 0 never split the tail tiles over K, 2 whenever possible
+    kOptPersist,         // OPMX_MOE_GEMM_PERSIST: 0 never the persistent form, 1 whenever possible
+    kNumOptions
+};
+int option(Option o);
+
+constexpr int kMaxDevices = 64;
+// The ordinal of the GPU that is current on this thread, or -1.
+inline int current_device()
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return -1;
+    return dev;
+}
+// Raises a kernel's dynamic shared-memory limit, once per GPU and kernel.  `done` is that kernel's
+// own bit mask of the GPUs already served.  Two threads that arrive together both set the
+// (same) attribute; neither launches before it is set.
+inline bool ensure_dynamic_smem(const void *kernel, int bytes, std::atomic<uint64_t> &done)
+{
+    const int dev = current_device();
+    if (dev < 0) return false;
+    const uint64_t bit = uint64_t{1} << dev;
+    if (done.load(std::memory_order_acquire) & bit) return true;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return false;
+    done.fetch_or(bit, std::memory_order_release);
+    return true;
+}
+// Compute units of the current GPU (looked up once per GPU), 0 on failure.
+int cu_count();
 
 #define OPMX_LAUNCH_CHECK()                                   \
     do {                                                      \

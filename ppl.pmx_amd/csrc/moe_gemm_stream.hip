@@ -237,13 +237,8 @@ int stream_launch_sw(const void *X, const int64_t *off, const void *W, const voi
     constexpr int smem = SW * ((SG || PAIR) ? 2 : 1) * 16 * RS + 2 * 16 * MT * RS;
     static_assert(!SGW || (SW / 2) * MT * 1024 <= smem, "the pair exchange reuses the staging memory");
     auto kern = gemm_stream_kernel<T, MT, KC, DEPTH, NT, SW, SG, PAIR, SGW>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                smem) != hipSuccess)
-            return OPMX_ERR_LAUNCH;
-        attr_done = true;
-    }
+    static std::atomic<uint64_t> attr_done{0};
+    if (!ensure_dynamic_smem(reinterpret_cast<const void *>(kern), smem, attr_done)) return OPMX_ERR_LAUNCH;
     dim3 grid(static_cast<unsigned>(ceil_div((SG || SGW) ? N / 2 : N, SROWS)),
               static_cast<unsigned>(max_mtiles(R, E, 16 * MT)));
     kern<<<grid, SW * 64, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),

@@ -286,7 +286,7 @@ inline int pick_gnx(int ntiles_n)
 {
     // XCD-grouped orders only when the n-tiles split evenly over the XCDs (else XCDs idle)
     int gnx = ntiles_n % 8 == 0 ? 8 : 16;
-    if (const char *v = std::getenv("OPMX_MOE_GEMM_GNX")) gnx = std::atoi(v);   // tuning knob
+    if (option(kOptGnx) >= 0) gnx = option(kOptGnx);   // tuning knob
     if (gnx != 0 && gnx != 4 && gnx != 8 && gnx != 16) gnx = 0;
     if (gnx == 4 && ntiles_n % 16 != 0) gnx = 0;
     if (gnx == 8 && ntiles_n % 8 != 0) gnx = 0;
@@ -1332,25 +1332,15 @@ int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B
     const int64_t nblocks = linear_ids(gnx, ntiles_m, ntiles_n);
     dim3 grid(static_cast<unsigned>(nblocks));
     dim3 block(WM * WN * 64);
-    static bool attr_done[2] = {false, false};
+    static std::atomic<uint64_t> attr_done[2];
     if (sw) {
         auto kern = gemm_tiled_kernel<T, BM, BN, WM, WN, true>;
-        if (!attr_done[1]) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    smem) != hipSuccess)
-                return OPMX_ERR_LAUNCH;
-            attr_done[1] = true;
-        }
+        if (!ensure_dynamic_smem(reinterpret_cast<const void *>(kern), smem, attr_done[1])) return OPMX_ERR_LAUNCH;
         kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
                                        static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_n, gnx);
     } else {
         auto kern = gemm_tiled_kernel<T, BM, BN, WM, WN, false>;
-        if (!attr_done[0]) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    smem) != hipSuccess)
-                return OPMX_ERR_LAUNCH;
-            attr_done[0] = true;
-        }
+        if (!ensure_dynamic_smem(reinterpret_cast<const void *>(kern), smem, attr_done[0])) return OPMX_ERR_LAUNCH;
         kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
                                        static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_n, gnx);
     }
@@ -1361,19 +1351,6 @@ int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B
 // Scratch memory of the tail launch of the direct-to-LDS kernel.
 constexpr int kSkCounters = 256;                  // tail tiles are fewer than the CUs
 constexpr int kSkTile = 256 * 256;                // elements of an output tile
-
-int cu_count()
-{
-    static int num_cu = 0;
-    if (num_cu == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-            return 0;
-        num_cu = n;
-    }
-    return num_cu;
-}
 
 // arrival counters, then one fp32 tile-sized slot per workgroup of the tail launch
 size_t sk_workspace_bytes(int cus)
@@ -1404,25 +1381,21 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
         sk_wgs = cus;
     // Measured: the exchange costs ~100 us against 1.43 us per k-tile.
     int sk_cost = 70;
-    if (const char *v = std::getenv("OPMX_MOE_GEMM_STREAMK")) {   // tuning knob: 0 = off, 2 = split whenever possible
-        if (std::atoi(v) == 0) sk_wgs = 0;
-        if (std::atoi(v) == 2) sk_cost = 0;
-    }
+    if (option(kOptStreamK) == 0) sk_wgs = 0;    // tuning knob: 0 = off, 2 = split whenever possible
+    if (option(kOptStreamK) == 2) sk_cost = 0;
     if (7 * (K / BK) <= 8 * sk_cost) sk_wgs = 0;     // sk_split() cannot split a K this short (g <= 8)
     int *sk_count = static_cast<int *>(ws);
     float *sk_part = reinterpret_cast<float *>(static_cast<char *>(ws) + kSkCounters * sizeof(int));
     dim3 grid(static_cast<unsigned>(dp_ids));
     dim3 block(256);
-    static bool attr_done[2] = {false, false};
-    if (!attr_done[sw ? 1 : 0]) {
+    static std::atomic<uint64_t> attr_done[2][2];
+    {
         const void *k1 = sw ? reinterpret_cast<const void *>(gemm_tiled_dlds_kernel<T, BM, BN, true, false>)
                             : reinterpret_cast<const void *>(gemm_tiled_dlds_kernel<T, BM, BN, false, false>);
         const void *k2 = sw ? reinterpret_cast<const void *>(gemm_tiled_dlds_kernel<T, BM, BN, true, true>)
                             : reinterpret_cast<const void *>(gemm_tiled_dlds_kernel<T, BM, BN, false, true>);
-        if (hipFuncSetAttribute(k1, hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess ||
-            hipFuncSetAttribute(k2, hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess)
+        if (!ensure_dynamic_smem(k1, smem, attr_done[sw ? 1 : 0][0]) || !ensure_dynamic_smem(k2, smem, attr_done[sw ? 1 : 0][1]))
             return OPMX_ERR_LAUNCH;
-        attr_done[sw ? 1 : 0] = true;
     }
     const T *Xp = static_cast<const T *>(X), *Wp = static_cast<const T *>(W), *Bp = static_cast<const T *>(B);
     T *Yp = static_cast<T *>(Y);
@@ -1433,14 +1406,14 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
     // workgroups of an XCD drift apart over the rounds and share less in L2 (+13 % HBM reads).
     bool persist = (gnx == 4 || gnx == 8 || gnx == 16) && K / BK >= 4 && ncols % 8 == 0 && reinterpret_cast<uintptr_t>(Y) % 16 == 0 &&
                    ncols * (2 * BM) < (int64_t{1} << 31) && cus >= 8 && cus % 8 == 0;
-    if (const char *v = std::getenv("OPMX_MOE_GEMM_PERSIST")) {   // tuning knob: 0 = never, 1 = whenever possible
-        if (std::atoi(v) == 0) persist = false;
+    if (option(kOptPersist) >= 0) {              // tuning knob: 0 = never, 1 = whenever possible
+        if (option(kOptPersist) == 0) persist = false;
     } else if (K / BK > 128) {
         persist = false;
     }
     if constexpr (BM == 256) if (persist) {
         const int smem_p = smem + 4 * 16 * (sw ? BN / 4 : BN / 2) * 2;       // + the four staging regions
-        static bool attr_p[4] = {false, false, false, false};
+        static std::atomic<uint64_t> attr_p[4];
         const bool hb = B != nullptr;
         using kernel_t = void (*)(const T *, const int64_t *, const T *, const T *, int, int64_t, int64_t, int64_t, T *, int,
                                   int, int, int);
@@ -1449,12 +1422,7 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
                                : (hb ? gemm_tiled_dlds_persist_kernel<T, BM, BN, false, true>
                                      : gemm_tiled_dlds_persist_kernel<T, BM, BN, false, false>);
         const int slot = (sw ? 2 : 0) + (hb ? 1 : 0);
-        if (!attr_p[slot]) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void *>(kp), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    smem_p) != hipSuccess)
-                return OPMX_ERR_LAUNCH;
-            attr_p[slot] = true;
-        }
+        if (!ensure_dynamic_smem(reinterpret_cast<const void *>(kp), smem_p, attr_p[slot])) return OPMX_ERR_LAUNCH;
         // ids congruent mod 8 stay on one XCD as long as the grid is a multiple of 8
         const unsigned wgs = static_cast<unsigned>(dp_ids < cus ? dp_ids : cus);
         if (sk_wgs > 0) sk_clear_kernel<<<1, 256, 0, s>>>(sk_count, kSkCounters);

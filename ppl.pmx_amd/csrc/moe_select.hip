@@ -570,15 +570,14 @@ int launch_moe_select(const void *X, const void *scores, int64_t T, int64_t H, i
 static __device__ __align__(256) unsigned char scratch[OPMX_MOE_SELECT_STATIC_SCRATCH_BYTES];
 
 namespace {
-constexpr int kMaxDevices = 64;
 std::mutex scratch_mutex;
 void *scratch_ptr[kMaxDevices];   // by device ordinal; written under scratch_mutex
 
 // The address of `scratch` on the GPU that is current on this thread (looked up once per GPU).
 int scratch_for_current_device(void **out)
 {
-    int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return OPMX_ERR_LAUNCH;
+    const int dev = current_device();
+    if (dev < 0) return OPMX_ERR_LAUNCH;
     std::lock_guard<std::mutex> hold(scratch_mutex);
     if (scratch_ptr[dev] == nullptr) {
         void *p = nullptr;

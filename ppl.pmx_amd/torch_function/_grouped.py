@@ -32,8 +32,10 @@ def grouped_linear(op, X, expert_offset, W, B, num_experts, epilogue=_lib.EPILOG
     off = expert_offset.to(torch.int64).contiguous()
     R = Xf.shape[0]
     n_out = N // 2 if epilogue == _lib.EPILOGUE_SWIGLU else N
-    # rows of one expert never exceed the token count when X is [*, k, K] from moe_select
-    hint = R // X.shape[-2] if X.dim() >= 3 and X.shape[-2] > 0 else 0
+    # No bound on the rows of one expert is passed: the operator accepts any [*, K] input, so the
+    # shape of X does not tell the token count, and the library then sizes its row tiles from
+    # twice the mean rows per expert (the smaller of the two bounds in nearly every routing anyway).
+    hint = 0
     Y = torch.empty(R, n_out, dtype=W.dtype, device=dev)
     L = _lib.lib()
     # optional scratch memory: with it the large-tile kernel balances its last rounds of tiles

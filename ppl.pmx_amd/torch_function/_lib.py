@@ -29,6 +29,7 @@ _i64, _int, _vp, _sz, _f = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes
 _SIGNATURES = {
     "opmx_moe_abi_version": (_int, []),
     "opmx_status_string": (ctypes.c_char_p, [_int]),
+    "opmx_moe_set_option": (_int, [ctypes.c_char_p, _int]),
     "opmx_linear": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp, _vp]),
     "opmx_moe_select_workspace_bytes": (_sz, [_i64, _int, _int]),
     "opmx_moe_select": (_int, [_vp, _vp, _i64, _i64, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
@@ -65,6 +66,14 @@ def lib():
             raise RuntimeError("libopmx_moe.so ABI version mismatch")
         _lib = handle
     return _lib
+
+
+def set_option(name: str, value) -> None:
+    """Sets a tuning knob of the grouped GEMMs (``opmx_moe_set_option``); ``None`` = automatic.
+    ``OPMX_MOE_GEMM`` also takes the words generic / tiled / stream."""
+    if name == "OPMX_MOE_GEMM" and isinstance(value, str) and not value.isdigit():
+        value = {"generic": 1, "tiled": 2, "stream": 3}[value]
+    check(lib().opmx_moe_set_option(name.encode(), -1 if value is None else int(value)), "opmx_moe_set_option")
 
 
 def check(status: int, what: str) -> None:

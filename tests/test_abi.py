@@ -91,6 +91,16 @@ def test_argument_validation_needs_no_device(lib):
     assert lib.opmx_moe_row_parallel_linear(None, None, None, None, 8, 0, 64, 32, 1, 0, None, None, 0, None) == 0
 
 
+def test_tuning_knobs(lib):
+    assert lib.opmx_moe_set_option(b"OPMX_MOE_GEMM", 2) == 0
+    assert lib.opmx_moe_set_option(b"OPMX_MOE_GEMM", -1) == 0          # back to automatic
+    for name in (b"OPMX_MOE_GEMM_TILED_VARIANT", b"OPMX_MOE_GEMM_STREAM_VARIANT", b"OPMX_MOE_GEMM_GNX",
+                 b"OPMX_MOE_GEMM_STREAMK", b"OPMX_MOE_GEMM_PERSIST"):
+        assert lib.opmx_moe_set_option(name, -1) == 0
+    assert lib.opmx_moe_set_option(b"OPMX_NO_SUCH_KNOB", 1) == -1
+    assert lib.opmx_moe_set_option(None, 1) == -1
+
+
 def test_workspace_sizes(lib):
     assert lib.opmx_moe_select_workspace_bytes(0, 8, 2) >= 256
     small = lib.opmx_moe_select_workspace_bytes(32, 8, 2)

@@ -32,12 +32,13 @@ def run_case(kind, sizes, K, N, dtype, bias, env=None, swiglu=False, lead3=False
     X = torch.randn(R, K, generator=g).to(dtype)
     W = (torch.randn(E, N, K, generator=g) * 0.05).to(dtype)
     B = torch.randn(E, N, generator=g).to(dtype) if bias else None
-    if lead3:                                  # [T, k, K] as MoeSelect returns it
+    if lead3 == "batch":                       # [1, R, K]: leading dimensions say nothing about the routing
+        X = X.view(1, R, K)
+    elif lead3:                                # [T, k, K] as MoeSelect returns it
         X = X.view(R // 2, 2, K)
-    old = {}
-    for key, val in (env or {}).items():
-        old[key] = os.environ.get(key)
-        os.environ[key] = val
+    from torch_function import _lib
+    for key, val in (env or {}).items():      # tuning knobs: force a kernel family / variant
+        _lib.set_option(key, val)
     try:
         args = (X.to(dev()), off.to(dev()), W.to(dev()), None if B is None else B.to(dev()))
         if swiglu:
@@ -48,11 +49,8 @@ def run_case(kind, sizes, K, N, dtype, bias, env=None, swiglu=False, lead3=False
             Y = OPMX.moe_row_parallel_linear(*args, None, E, K, N, True)
         torch.cuda.synchronize()
     finally:
-        for key, val in old.items():
-            if val is None:
-                os.environ.pop(key, None)
-            else:
-                os.environ[key] = val
+        for key in (env or {}):
+            _lib.set_option(key, None)         # back to automatic
     ref = O.moe_column_parallel_linear(X, off, W, B, acc=torch.float64, out_dtype=torch.float64)
     if swiglu:
         ref = O.swiglu(ref, acc=torch.float64)
@@ -200,9 +198,12 @@ def test_stream_kernel_variants(variant, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 def test_automatic_selection_and_hint(dtype):
-    # [T, k, K] input: the wrapper passes rows-per-expert hint T
+    # [T, k, K] input, as MoeSelect returns it
     run_case("column", [10, 6, 0, 16, 8, 8, 9, 7], 512, 256, dtype, False, lead3=True)
     run_case("column", [700, 6, 0, 16, 800, 8, 90, 428], 512, 256, dtype, False, lead3=True)
+    # a 3-D input that is not [T, k, K]: experts with thousands of rows behind a leading 1
+    run_case("column", [1500, 6, 0, 1600, 800, 8, 90, 428], 512, 256, dtype, False, lead3="batch")
+    run_case("row", [40, 6, 0, 16, 80, 8, 90, 16], 512, 256, dtype, False, lead3="batch")
     run_case("row", [700, 6, 0, 16, 800, 8, 90, 428], 512, 256, dtype, True)
     if dtype != torch.float32:
         # K a multiple of 8 but not of 64 with many rows: the stream kernel's 128-row tiles, not the FMA fallback

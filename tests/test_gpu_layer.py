@@ -41,6 +41,24 @@ def run_ops(x, Wg, wu, w2, E, k, bias=None, route=False):
     return dict(scores=scores, x_expand=xe, weights=w, inv=inv, off=off, x13=x13, act=act, y=y, out=out)
 
 
+def check_output(out, scores, host, E, k, full=True, sample=48):
+    """Layer output against the fp32-accumulated oracle routed by the same low-precision scores:
+    the whole oracle layer, or (large configurations) the permutation-free float64 formulation
+    on a sample of tokens."""
+    x, Wg, wu, w2 = host
+    out = out.cpu().double()
+    if full:
+        ref = O.moe_layer(x, Wg, wu, w2, E, k, scores=scores, round_between_ops=False).double()
+        err = (out - ref).abs()
+    else:
+        T = x.shape[0]
+        pick = torch.randperm(T, generator=torch.Generator().manual_seed(1))[:sample]
+        ref = O.moe_layer_dense_fp64(x[pick], Wg, wu, w2, E, k, scores=scores[pick])
+        err = (out[pick] - ref).abs()
+    assert float(err.max()) <= MAX_ABS and float(err.mean()) <= MEAN_ABS, (float(err.max()), float(err.mean()))
+    return float(err.max()), float(err.mean())
+
+
 def check_against_oracle(g, host, E, k, bias=None, full=True, sample=48):
     x, Wg, wu, w2 = host
     scores = g["scores"].cpu()
@@ -53,19 +71,14 @@ def check_against_oracle(g, host, E, k, bias=None, full=True, sample=48):
     assert torch.equal(g["off"].cpu(), roff)
     assert torch.equal(g["inv"].cpu(), rinv)
     assert torch.equal(g["x_expand"].cpu(), rxe)
-    out = g["out"].cpu().double()
-    if full:
-        ref = O.moe_layer(x, Wg, wu, w2, E, k, scores=scores, round_between_ops=False).double()
-        err = (out - ref).abs()
-        assert float(err.max()) <= MAX_ABS and float(err.mean()) <= MEAN_ABS, (float(err.max()), float(err.mean()))
-        return float(err.max()), float(err.mean())
-    # large configs: the permutation-free float64 formulation on a sample of tokens
-    T = x.shape[0]
-    pick = torch.randperm(T, generator=torch.Generator().manual_seed(1))[:sample]
-    ref = O.moe_layer_dense_fp64(x[pick], Wg, wu, w2, E, k, scores=scores[pick])
-    err = (out[pick] - ref).abs()
-    assert float(err.max()) <= MAX_ABS and float(err.mean()) <= MEAN_ABS, (float(err.max()), float(err.mean()))
-    return float(err.max()), float(err.mean())
+    return check_output(g["out"], scores, host, E, k, full=full, sample=sample)
+
+
+def check_fused_against_oracle(layer_out, g, host, E, k, full=True):
+    """A fused form of the block (SwiGLU in the GEMM epilogue, router gate + select in one call)
+    against the ORACLE, not against the operator-by-operator GPU result: routed by the logits
+    the separate router gate returned (the fused block computes the same ones)."""
+    return check_output(layer_out, g["scores"].cpu(), host, E, k, full=full)
 
 
 def test_tiny_config_fp32():
@@ -97,13 +110,15 @@ def test_mixtral_8x7b_decode(mixtral_8x7b, T):
     m = build_layer(4096, 14336, 8, 2, torch.float16, Wg, wu, w2)
     assert torch.equal(m(x[:T]), g["out"])
     mf = build_layer(4096, 14336, 8, 2, torch.float16, Wg, wu, w2, fuse=True)
-    err = (mf(x[:T]).double() - g["out"].double()).abs()
-    assert float(err.max()) <= MAX_ABS and float(err.mean()) <= MEAN_ABS
+    check_fused_against_oracle(mf(x[:T]), g, (host[0][:T],) + host[1:], 8, 2)
     # router gate and select in one launch: the same bar on the logits that launch returns
     gr = run_ops(x[:T], Wg, wu, w2, 8, 2, route=True)
     check_against_oracle(gr, (host[0][:T],) + host[1:], 8, 2)
     mr = build_layer(4096, 14336, 8, 2, torch.float16, Wg, wu, w2, route=True)
     assert torch.equal(mr(x[:T]), gr["out"])
+    # both fused forms together, against the oracle routed by the fused call's logits
+    mfr = build_layer(4096, 14336, 8, 2, torch.float16, Wg, wu, w2, fuse=True, route=True)
+    check_fused_against_oracle(mfr(x[:T]), gr, (host[0][:T],) + host[1:], 8, 2)
 
 
 @pytest.mark.parametrize("T,full", [(2048, True), (8192, False)])
@@ -115,10 +130,10 @@ def test_mixtral_8x7b_prefill_skewed(mixtral_8x7b, T, full):
     counts = (g["off"][1:] - g["off"][:-1]).cpu()
     assert float(counts.max()) / (T * k) > 0.40, counts.tolist()
     check_against_oracle(g, (host[0][:T],) + host[1:], E, k, bias=bias, full=full)
-    mf = build_layer(4096, 14336, E, k, torch.float16, Wg, wu, w2, fuse=True)
-    mf.gate.bias = torch.nn.Parameter(bias.to(dev()), requires_grad=False)
-    err = (mf(x[:T]).double() - g["out"].double()).abs()
-    assert float(err.max()) <= MAX_ABS and float(err.mean()) <= MEAN_ABS
+    for route in (False, True):     # SwiGLU in the GEMM epilogue, alone and with the fused router call
+        mf = build_layer(4096, 14336, E, k, torch.float16, Wg, wu, w2, fuse=True, route=route)
+        mf.gate.bias = torch.nn.Parameter(bias.to(dev()), requires_grad=False)
+        check_fused_against_oracle(mf(x[:T]), g, (host[0][:T],) + host[1:], E, k, full=full)
     # size-independent property: the layer is row-wise, so a row subset gives the same rows
     # up to the tile a row lands in (accumulation order inside a row is fixed => bit equal)
     sub = run_ops(x[:64], Wg, wu, w2, E, k, bias=bias.to(dev()))
@@ -132,6 +147,9 @@ def test_fine_grained_64_experts_bf16(T):
     (x, Wg, wu, w2), host = gpu_inputs(T, H, E, I, torch.bfloat16, seed=3)
     g = run_ops(x, Wg, wu, w2, E, k)
     check_against_oracle(g, host, E, k)
+    for route in (False, True):
+        mf = build_layer(H, I, E, k, torch.bfloat16, Wg, wu, w2, fuse=True, route=route)
+        check_fused_against_oracle(mf(x), g, host, E, k)
 
 
 @pytest.mark.parametrize("T,full", [(16, True), (4096, False)])
@@ -140,3 +158,5 @@ def test_mixtral_8x22b_shape(T, full):
     (x, Wg, wu, w2), host = gpu_inputs(T, H, E, I, torch.float16, seed=4)
     g = run_ops(x, Wg, wu, w2, E, k)
     check_against_oracle(g, host, E, k, full=full)
+    mf = build_layer(H, I, E, k, torch.float16, Wg, wu, w2, fuse=True)
+    check_fused_against_oracle(mf(x), g, host, E, k, full=full)

@@ -76,6 +76,34 @@ def nodes_of(graph):
     return found
 
 
+def test_symbolics_match_the_reference_fixture():
+    """Node kind, input / output counts and attribute names and values of every operator against
+    tests/golden/reference_symbolics.json, which tests/golden/make_symbolic_fixture.py wrote by
+    exporting the same calls through the reference's own torch_function package (MoeSelect.py:5-17,
+    MoeColumnParallelLinear.py:8-27, MoeRowParallelLinear.py:8-26, MoeReduce.py:5-12, SwiGLU.py:5-8,
+    SiLU.py, Linear.py:7-22, RMSNorm.py:6-11,29-39)."""
+    import json
+    import os
+    import sys
+    golden = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    sys.path.insert(0, golden)
+    try:
+        from symbolic_cases import cases, export_nodes
+    finally:
+        sys.path.remove(golden)
+    want = json.load(open(os.path.join(golden, "reference_symbolics.json")))["nodes"]
+    mine = cases(OPMX)
+    assert sorted(want) == sorted(name for name, _, _ in mine)
+    for name, mod, args in mine:
+        got = export_nodes(mod, args)
+        assert len(got) == len(want[name]) >= 1, name
+        for g, w in zip(got, want[name]):
+            assert g[:3] == w[:3], (name, g, w)
+            assert sorted(g[3]) == sorted(w[3]), (name, g[3], w[3])
+            for key, val in w[3].items():
+                assert abs(g[3][key] - val) <= 1e-9 * max(1.0, abs(val)), (name, key, g[3][key], val)
+
+
 @pytest.mark.parametrize("fused,bias", [(True, False), (False, True)])
 def test_mixtral_block_exports_reference_nodes(fused, bias):
     H, I, E, k = 64, 96, 8, 2

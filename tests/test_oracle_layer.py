@@ -41,6 +41,30 @@ def test_grouped_linear_special_cases():
     assert Y3.shape == (4, 2, N)
 
 
+def test_linear_with_bias_pins():
+    """O.linear (Linear.py:32) against the library routine and against an explicit double loop,
+    with a bias whose sign, index and transposition mistakes would all show."""
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(11)
+    X, W, B = torch.randn(5, 7, generator=g), torch.randn(3, 7, generator=g), torch.tensor([10.0, -20.0, 30.0])
+    got = O.linear(X, W, B)
+    assert got.shape == (5, 3)
+    assert torch.allclose(got, F.linear(X, W, B), rtol=0, atol=1e-5)
+    for t in range(5):
+        for n in range(3):
+            want = sum(float(X[t, c]) * float(W[n, c]) for c in range(7)) + float(B[n])
+            assert abs(float(got[t, n]) - want) < 1e-4
+    assert torch.allclose(O.linear(X, W), F.linear(X, W), rtol=0, atol=1e-5)       # no bias
+    # known answer: ones . arange + bias
+    assert torch.equal(O.linear(torch.ones(1, 4), torch.arange(8.0).view(2, 4), torch.tensor([0.5, -0.5])),
+                       torch.tensor([[6.5, 21.5]]))
+    # low precision: fp32 accumulation, rounded once, in the weight's dtype; leading dims kept
+    Xh, Wh, Bh = torch.randn(2, 3, 64, generator=g).half(), torch.randn(9, 64, generator=g).half(), torch.randn(9, generator=g).half()
+    got = O.linear(Xh, Wh, Bh)
+    assert got.dtype == torch.float16 and got.shape == (2, 3, 9)
+    assert torch.equal(got, F.linear(Xh.float(), Wh.float(), Bh.float()).half())
+
+
 def test_grouped_linear_low_precision_rounds_once():
     g = torch.Generator().manual_seed(2)
     E, N, K, R = 2, 8, 512, 6
