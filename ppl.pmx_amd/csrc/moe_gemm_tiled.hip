@@ -700,6 +700,17 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t raw_descriptor(const void *bas
                                              static_cast<int>(0xFFFFFFFFu), 0x00020000);
 }
 
+// Descriptor over `bytes` bytes from `base` (both uniform): accesses at offsets >= bytes are
+// dropped by the hardware range check.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t bounded_descriptor(const void *base, uint32_t bytes)
+{
+    const uint64_t b = reinterpret_cast<uint64_t>(base);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(b));
+    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(b >> 32));
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>((static_cast<uint64_t>(hi) << 32) | lo), 0,
+                                             static_cast<int>(__builtin_amdgcn_readfirstlane(bytes)), 0x00020000);
+}
+
 // 16 bytes per lane from descriptor + soff + voff straight into LDS at lds + 16*lane (lds is
 // wave-uniform).
 __device__ __forceinline__ void load_to_lds_16(__amdgpu_buffer_rsrc_t r, char *lds, uint32_t voff, int soff)
@@ -710,20 +721,23 @@ __device__ __forceinline__ void load_to_lds_16(__amdgpu_buffer_rsrc_t r, char *l
 // This lane's share of the sixteen 1 KiB wave loads per operand and k-tile: load i of wave w
 // fetches tile rows 8*(w*L+i) .. +7, lane l the 16-byte chunk of row 8*(w*L+i) + l/8 that
 // belongs in LDS slot l%8 of that row (slots are XOR-swizzled by row).  Results are byte offsets
-// from the tile's X rows / the expert's W at k = 0; rows past the tile or the matrix repeat the
-// last valid row (they feed accumulators that are never stored).  With SWIGLU a wave's WTN
-// W-rows are WTN/2 gate rows followed by the WTN/2 up rows of the same output columns.
+// from the tile's X rows / the expert's W at k = 0.  W rows past the matrix repeat the last valid
+// row (they feed accumulators that are never stored).  X rows past the tile keep their own
+// offset: the tile's descriptor ends with its last row (x_descriptor), so the range check
+// answers those loads with zeros -- the MFMAs of a ragged tile's missing rows then multiply
+// zeros, which costs far less power than multiplying a copy of real data, and the part runs its
+// MFMA kernels against a power limit.  With SWIGLU a wave's WTN W-rows are WTN/2 gate rows
+// followed by the WTN/2 up rows of the same output columns.
 template <int LA, int LB, int WTN, bool SWIGLU>
-__device__ __forceinline__ void tile_sources(int rows, int64_t n0, int64_t K, int64_t N, int64_t ncols, int wave,
+__device__ __forceinline__ void tile_sources(int /*rows*/, int64_t n0, int64_t K, int64_t N, int64_t ncols, int wave,
                                              int lane, uint32_t (&a_src)[LA], uint32_t (&b_src)[LB])
 {
     const int lrow8 = lane >> 3, slot = lane & 7;
 #pragma unroll
     for (int i = 0; i < LA; ++i) {
         const int row = (wave * LA + i) * 8 + lrow8;
-        const int r = row < rows ? row : rows - 1;
         const int c = slot ^ ((row >> 1) & 7);
-        a_src[i] = static_cast<uint32_t>((r * K + c * 8) * 2);
+        a_src[i] = static_cast<uint32_t>((row * K + c * 8) * 2);
     }
 #pragma unroll
     for (int i = 0; i < LB; ++i) {
@@ -740,6 +754,14 @@ __device__ __forceinline__ void tile_sources(int rows, int64_t n0, int64_t K, in
         const int c = slot ^ ((row >> 1) & 7);
         b_src[i] = static_cast<uint32_t>((wrow * K + c * 8) * 2);
     }
+}
+
+// Descriptor of a tile's X rows: `rows` rows of K elements from row `row0` on, and nothing behind
+// them (loads of the rows a ragged tile lacks return zeros, see tile_sources).
+template <typename T>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t x_descriptor(const T *X, int64_t row0, int rows, int64_t K)
+{
+    return bounded_descriptor(X + row0 * K, static_cast<uint32_t>(rows * K * 2));
 }
 
 // Where a workgroup starts its walk over the nk k-tiles (it wraps around): an eighth of K further
@@ -875,7 +897,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
     const int64_t n0 = static_cast<int64_t>(tile_n) * BNO;
-    const __amdgpu_buffer_rsrc_t rx = raw_descriptor(X + mt.row0 * K);
+    const __amdgpu_buffer_rsrc_t rx = x_descriptor(X, mt.row0, mt.rows, K);
     const __amdgpu_buffer_rsrc_t rw = raw_descriptor(W + static_cast<int64_t>(mt.e) * N * K);
 
     uint32_t a_src[LA], b_src[LB];     // byte offsets from the tile's X / W base at k = 0
@@ -1034,16 +1056,6 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
         tile_epilogue<T, WTM, WTN, SWIGLU>(acc, Bias, Y, mt, N, ncols, n0, wm, wn, lane);
 }
 
-// Descriptor over `bytes` bytes from `base` (both uniform): accesses at offsets >= bytes are
-// dropped by the hardware range check.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t bounded_descriptor(const void *base, uint32_t bytes)
-{
-    const uint64_t b = reinterpret_cast<uint64_t>(base);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(b));
-    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(b >> 32));
-    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>((static_cast<uint64_t>(hi) << 32) | lo), 0,
-                                             static_cast<int>(__builtin_amdgcn_readfirstlane(bytes)), 0x00020000);
-}
 __device__ __forceinline__ void store_16(__amdgpu_buffer_rsrc_t r, uint32_t voff, u32x4 v)
 {
     __builtin_amdgcn_raw_buffer_store_b128(v, r, voff, 0, 0);
@@ -1211,7 +1223,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
     int cur_n;
     locate_any(id, gnx, mtiles, ntiles_n, off != nullptr, s_off, E, R, BM, cur, cur_n);
     if (cur.rows == 0) return;
-    __amdgpu_buffer_rsrc_t rx = raw_descriptor(X + cur.row0 * K);
+    __amdgpu_buffer_rsrc_t rx = x_descriptor(X, cur.row0, cur.rows, K);
     __amdgpu_buffer_rsrc_t rw = raw_descriptor(W + static_cast<int64_t>(cur.e) * N * K);
     uint32_t a_src[LA], b_src[LB];
     tile_sources<LA, LB, WTN, SWIGLU>(cur.rows, static_cast<int64_t>(cur_n) * BNO, K, N, ncols, wave, lane, a_src, b_src);
@@ -1271,7 +1283,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
         b ^= 1;
         for (int kt = 1; kt + 2 < nk; ++kt, b ^= 1) OPMX_ITERX(kt + 2, b, true, true, false, 16);
         // all loads of this tile are issued: retarget the load state, then stream on
-        rx = raw_descriptor(X + nxt.row0 * K);
+        rx = x_descriptor(X, nxt.row0, nxt.rows, K);
         rw = raw_descriptor(W + static_cast<int64_t>(nxt.e) * N * K);
         tile_sources<LA, LB, WTN, SWIGLU>(nxt.rows, static_cast<int64_t>(nxt_n) * BNO, K, N, ncols, wave, lane, a_src, b_src);
         const int64_t nw0 = static_cast<int64_t>(cur_n) * BNO + wn * (SWIGLU ? WTN / 2 : WTN);   // first output column of this wave
