@@ -134,6 +134,9 @@ def main():
     ap.add_argument("--fuse-router-select", action="store_true",
                     help="router gate and MoeSelect through the fused call (one launch up to 8 tokens)")
     ap.add_argument("--fuse-swiglu", action="store_true", help="apply SwiGLU in the gate/up GEMM epilogue")
+    ap.add_argument("--fuse-gather", action="store_true",
+                    help="MoeSelect returns an index instead of the expanded copy of the tokens; the gate/up GEMM "
+                         "reads its rows through it")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg")
     ap.add_argument("--no-device-ceilings", action="store_true",
@@ -222,6 +225,30 @@ def main():
         layer.gate.bias = torch.nn.Parameter(bias, requires_grad=False)
     Wg, wu, w2, gb = layer.gate.weight, layer.wu.weight, layer.w2.weight, layer.gate.bias
 
+    # router gate and MoeSelect in the form the flags ask for -> (xe, w, inv, off); with --fuse-gather
+    # `xe` is the index that stands for the expanded copy
+    def timed_select(timed):
+        if args.fuse_gather:
+            if args.fuse_router_select:
+                w, inv, off, rt, sc = timed("router_and_select", lambda: OPMX.moe_route_select_index(x, Wg, gb, E, k))
+            else:
+                sc = timed("router_linear", lambda: OPMX.linear(x, Wg, gb, H, E))
+                w, inv, off, rt = timed("moe_select", lambda: OPMX.moe_select_index(sc, E, k))
+            return rt, w, inv, off
+        if args.fuse_router_select:
+            xe, w, inv, off, sc = timed("router_and_select", lambda: OPMX.moe_route_select(x, Wg, gb, E, k))
+        else:
+            sc = timed("router_linear", lambda: OPMX.linear(x, Wg, gb, H, E))
+            xe, w, inv, off = timed("moe_select", lambda: OPMX.moe_select(x, sc, E, k))
+        return xe, w, inv, off
+
+    def gemm1(xe, off):
+        if args.fuse_gather:
+            return OPMX.moe_column_parallel_linear_indexed(x, xe, off, wu, None, E, H, 2 * I, swiglu=args.fuse_swiglu)
+        if args.fuse_swiglu:
+            return OPMX.moe_column_parallel_linear_swiglu(xe, off, wu, None, E, H, 2 * I)
+        return OPMX.moe_column_parallel_linear(xe, off, wu, None, None, E, H, 2 * I, False)
+
     # ---- one instrumented pass: routing statistics + per-operator durations
     def ops(record=None):
         def timed(name, fn):
@@ -233,26 +260,18 @@ def main():
             b.record()
             record.append((name, a, b))
             return r
-        if args.fuse_router_select:
-            xe, w, inv, off, sc = timed("router_and_select", lambda: OPMX.moe_route_select(x, Wg, gb, E, k))
-        else:
-            sc = timed("router_linear", lambda: OPMX.linear(x, Wg, gb, H, E))
-            xe, w, inv, off = timed("moe_select", lambda: OPMX.moe_select(x, sc, E, k))
+        xe, w, inv, off = timed_select(timed)
         if args.fuse_swiglu:
-            act = timed("gate_up_gemm", lambda: OPMX.moe_column_parallel_linear_swiglu(xe, off, wu, None, E, H, 2 * I))
+            act = timed("gate_up_gemm", lambda: gemm1(xe, off))
         else:
-            h = timed("gate_up_gemm", lambda: OPMX.moe_column_parallel_linear(xe, off, wu, None, None, E, H, 2 * I, False))
+            h = timed("gate_up_gemm", lambda: gemm1(xe, off))
             act = timed("swiglu", lambda: OPMX.swiglu(h))
         y = timed("down_gemm", lambda: OPMX.moe_row_parallel_linear(act, off, w2, None, None, E, I, H, True))
         out = timed("moe_reduce", lambda: OPMX.moe_reduce(y, w, inv, k))
         return out, off
 
     def step(i=-1, ev=None, stride=1):
-        if args.fuse_router_select:
-            xe, w, inv, off, sc = OPMX.moe_route_select(x, Wg, gb, E, k)
-        else:
-            sc = OPMX.linear(x, Wg, gb, H, E)
-            xe, w, inv, off = OPMX.moe_select(x, sc, E, k)
+        xe, w, inv, off = timed_select(lambda name, fn: fn())
         mark = ev is not None and i % stride == 0
         if mark:
             ev[i // stride][0].record()
@@ -271,10 +290,6 @@ def main():
             step(i, ev, stride)
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / n * 1e3
-
-    gemm1 = (lambda xe, off: OPMX.moe_column_parallel_linear_swiglu(xe, off, wu, None, E, H, 2 * I)) \
-        if args.fuse_swiglu else \
-        (lambda xe, off: OPMX.moe_column_parallel_linear(xe, off, wu, None, None, E, H, 2 * I, False))
 
     with torch.inference_mode():
         out, off = ops()
@@ -424,7 +439,8 @@ def main():
         "config": {"workload": "{} MoE layer {}, T={} tokens, hidden={}, experts={}, top-{}, ffn={}, TP=1".format(
             cfg["name"], "decode" if hbm_bound else "prefill", T, H, E, k, I),
             "path": "drop-in operator sequence" + (" + fused SwiGLU epilogue" if args.fuse_swiglu else "")
-            + (" + router gate and select in one call" if args.fuse_router_select else ""),
+            + (" + router gate and select in one call" if args.fuse_router_select else "")
+            + (" + token gather folded into the gate/up GEMM" if args.fuse_gather else ""),
             "active_experts": active, "max_expert_share": round(float(counts.max()) / R, 3)},
         "roofline": roof, "layer": lay,
         "hip_graph_replay": None if graph_ms is None else {"ms_per_step": round(graph_ms, 4),

@@ -146,6 +146,23 @@ int opmx_moe_route_select(const void *X, const void *gate_weight, const void *ga
                           void *expert_weights, int64_t *invert_permutation, int64_t *expert_offset,
                           int32_t *expert_ids, void *workspace, size_t workspace_bytes, void *stream);
 
+/* MoeSelect without the row copy (torch_function/MoeSelect.py:37-64 except :45-47): the routing
+ * outputs of opmx_moe_select -- expert_weights, invert_permutation, expert_offset, bit for bit
+ * the same -- and, instead of X_expand_permute, the index that stands for it:
+ *   row_token [T*k] int32: row r of X_expand_permute would be X[row_token[r], :]
+ *                          (row_token[invert_permutation[t*k+s]] = t; perm[r] / k in the reference's terms).
+ * opmx_moe_column_parallel_linear_indexed reads X through it, so the [T*k, H] copy is never
+ * written or read.  Limits and workspace are those of opmx_moe_select.
+ * opmx_moe_route_select_index is the same with the router gate in front (see
+ * opmx_moe_route_select): scores [T,E] is then an output. */
+int opmx_moe_select_index(const void *scores, int64_t T, int E, int k, int dtype, void *expert_weights,
+                          int64_t *invert_permutation, int64_t *expert_offset, int32_t *row_token,
+                          int32_t *expert_ids, void *workspace, size_t workspace_bytes, void *stream);
+int opmx_moe_route_select_index(const void *X, const void *gate_weight, const void *gate_bias, int64_t T,
+                                int64_t H, int E, int k, int dtype, void *scores, void *expert_weights,
+                                int64_t *invert_permutation, int64_t *expert_offset, int32_t *row_token,
+                                int32_t *expert_ids, void *workspace, size_t workspace_bytes, void *stream);
+
 /* Grouped expert GEMM.  Replaces the per-expert F.linear loops of
  * MoeColumnParallelLinear.forward (torch_function/MoeColumnParallelLinear.py:58-69)
  * and MoeRowParallelLinear.forward (torch_function/MoeRowParallelLinear.py:44-60)
@@ -168,6 +185,17 @@ int opmx_moe_column_parallel_linear(const void *X, const int64_t *expert_offset,
                                     const void *B, int E, int64_t R, int64_t K, int64_t N,
                                     int dtype, int epilogue, int64_t rows_per_expert_hint,
                                     void *Y, void *workspace, size_t workspace_bytes, void *stream);
+/* opmx_moe_column_parallel_linear with its rows read through an index: GEMM row r is
+ * X[row_index[r], :] with X [X_rows, K] (the tokens, not their expanded copies) and row_index
+ * [R] int32 with values in [0, X_rows) -- the row_token output of opmx_moe_select_index.  Equals
+ * opmx_moe_column_parallel_linear on X_expand_permute bit for bit (the reference gathers first,
+ * torch_function/MoeSelect.py:45-47, then multiplies, MoeColumnParallelLinear.py:58-67).
+ * fp16 / bf16 kernels need X_rows * K * 2 < 2^31 (else the fp32-style fallback kernel runs). */
+int opmx_moe_column_parallel_linear_indexed(const void *X, int64_t X_rows, const int32_t *row_index,
+                                            const int64_t *expert_offset, const void *W, const void *B, int E,
+                                            int64_t R, int64_t K, int64_t N, int dtype, int epilogue,
+                                            int64_t rows_per_expert_hint, void *Y, void *workspace,
+                                            size_t workspace_bytes, void *stream);
 int opmx_moe_row_parallel_linear(const void *X, const int64_t *expert_offset, const void *W,
                                  const void *B, int E, int64_t R, int64_t K, int64_t N,
                                  int dtype, int64_t rows_per_expert_hint,

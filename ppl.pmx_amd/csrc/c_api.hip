@@ -87,13 +87,15 @@ size_t grouped_gemm_workspace_bytes(int E, int64_t R, int64_t K, int64_t N, int 
 
 int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
                         int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint, void *Y, void *ws,
-                        size_t ws_bytes, hipStream_t s)
+                        size_t ws_bytes, hipStream_t s, RowGather g)
 {
     const int64_t ncols = epilogue == OPMX_EPILOGUE_SWIGLU ? N / 2 : N;
     if (R == 0 || ncols == 0) return OPMX_OK;
     const bool lowp = dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16;
+    // (through a row index the MFMA kernels address X with 32-bit byte offsets)
     const bool mfma_ok = lowp && K > 0 && K % 8 == 0 && aligned16(X) && aligned16(W) &&
-                         N * K < (int64_t{1} << 31) && R * K < (int64_t{1} << 40);
+                         N * K < (int64_t{1} << 31) && R * K < (int64_t{1} << 40) &&
+                         (g.index == nullptr || g.x_rows * K * 2 < (int64_t{1} << 31));
     const bool tiled_ok = mfma_ok && K % 64 == 0;
     // Row-tile sizing: twice the mean rows per expert, never above what the caller can
     // guarantee.  An expert with more rows than one tile simply takes several tiles.
@@ -114,7 +116,7 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
 
     if (choice == 3)
         return launch_gemm_stream(X, off, W, B, E, R, K, N, dtype, epilogue, hint,
-                                  option(kOptStreamVariant) < 0 ? 0 : option(kOptStreamVariant), Y, s);
+                                  option(kOptStreamVariant) < 0 ? 0 : option(kOptStreamVariant), Y, s, g);
     if (choice == 2) {
         // The direct-to-LDS kernel takes 256x256 tiles unless they would fill the CUs less than
         // twice (the Mixtral down projection at T=2048: 1.3 rounds) or the experts hold fewer than
@@ -124,9 +126,9 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
         const int64_t tiles256 = (R / 256 + (E + 1) / 2) * ((out_cols + 255) / 256);
         const int dflt = R / E >= 128 && tiles256 >= 512 ? 0 : 3;
         return launch_gemm_tiled(X, off, W, B, E, R, K, N, dtype, epilogue,
-                                 option(kOptTiledVariant) < 0 ? dflt : option(kOptTiledVariant), Y, ws, ws_bytes, s);
+                                 option(kOptTiledVariant) < 0 ? dflt : option(kOptTiledVariant), Y, ws, ws_bytes, s, g);
     }
-    return launch_gemm_generic(X, off, W, B, E, R, K, N, dtype, epilogue, Y, s);
+    return launch_gemm_generic(X, off, W, B, E, R, K, N, dtype, epilogue, Y, s, g);
 }
 
 }  // namespace opmx
@@ -224,6 +226,40 @@ int opmx_moe_route_select(const void *X, const void *gate_weight, const void *ga
                                    expert_weights, invert_permutation, expert_offset, expert_ids, workspace, st(stream));
 }
 
+int opmx_moe_select_index(const void *scores, int64_t T, int E, int k, int dtype, void *expert_weights,
+                          int64_t *invert_permutation, int64_t *expert_offset, int32_t *row_token,
+                          int32_t *expert_ids, void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (T < 0 || E <= 0 || k <= 0 || k > E) return OPMX_ERR_BAD_ARGUMENT;
+    if (!dtype_ok(dtype) || E > OPMX_MOE_MAX_EXPERTS || k > OPMX_MOE_MAX_EXPERTS_PER_TOKEN)
+        return OPMX_ERR_UNSUPPORTED;
+    if (T > (int64_t{1} << 31) / k) return OPMX_ERR_UNSUPPORTED;
+    if (!expert_offset) return OPMX_ERR_BAD_ARGUMENT;
+    if (T > 0 && (!scores || !expert_weights || !invert_permutation || !row_token)) return OPMX_ERR_BAD_ARGUMENT;
+    if (T > 0 && (!workspace || workspace_bytes < moe_select_workspace_bytes(T, E, k))) return OPMX_ERR_WORKSPACE;
+    if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 255u)) return OPMX_ERR_ALIGNMENT;
+    return launch_moe_select(nullptr, scores, T, 0, E, k, dtype, nullptr, expert_weights, invert_permutation,
+                             expert_offset, expert_ids, workspace, st(stream), row_token);
+}
+
+int opmx_moe_route_select_index(const void *X, const void *gate_weight, const void *gate_bias, int64_t T, int64_t H,
+                                int E, int k, int dtype, void *scores, void *expert_weights,
+                                int64_t *invert_permutation, int64_t *expert_offset, int32_t *row_token,
+                                int32_t *expert_ids, void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (T < 0 || H < 0 || E <= 0 || k <= 0 || k > E) return OPMX_ERR_BAD_ARGUMENT;
+    if (!dtype_ok(dtype) || E > OPMX_MOE_MAX_EXPERTS || k > OPMX_MOE_MAX_EXPERTS_PER_TOKEN)
+        return OPMX_ERR_UNSUPPORTED;
+    if (T > (int64_t{1} << 31) / k) return OPMX_ERR_UNSUPPORTED;
+    if (!expert_offset) return OPMX_ERR_BAD_ARGUMENT;
+    if (T > 0 && (!scores || !expert_weights || !invert_permutation || !row_token)) return OPMX_ERR_BAD_ARGUMENT;
+    if (T > 0 && H > 0 && (!X || !gate_weight)) return OPMX_ERR_BAD_ARGUMENT;
+    if (T > 0 && (!workspace || workspace_bytes < moe_select_workspace_bytes(T, E, k))) return OPMX_ERR_WORKSPACE;
+    if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 255u)) return OPMX_ERR_ALIGNMENT;
+    return launch_moe_route_select(X, gate_weight, gate_bias, T, H, E, k, dtype, scores, nullptr, expert_weights,
+                                   invert_permutation, expert_offset, expert_ids, workspace, st(stream), row_token);
+}
+
 size_t opmx_moe_grouped_gemm_workspace_bytes(int E, int64_t R, int64_t K, int64_t N, int dtype)
 {
     return grouped_gemm_workspace_bytes(E, R, K, N, dtype);
@@ -231,7 +267,7 @@ size_t opmx_moe_grouped_gemm_workspace_bytes(int E, int64_t R, int64_t K, int64_
 
 static int grouped_checked(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
                            int64_t K, int64_t N, int dtype, int epilogue, int64_t hint, void *Y, void *ws,
-                           size_t ws_bytes, void *stream)
+                           size_t ws_bytes, void *stream, RowGather g = {})
 {
     if (E <= 0 || R < 0 || K < 0 || N < 0) return OPMX_ERR_BAD_ARGUMENT;
     if (!dtype_ok(dtype) || E > OPMX_MOE_MAX_EXPERTS) return OPMX_ERR_UNSUPPORTED;
@@ -239,7 +275,7 @@ static int grouped_checked(const void *X, const int64_t *off, const void *W, con
     if (epilogue == OPMX_EPILOGUE_SWIGLU && N % 2) return OPMX_ERR_BAD_ARGUMENT;
     if (R == 0 || N == 0) return OPMX_OK;
     if (!X || !off || !W || !Y || K == 0) return OPMX_ERR_BAD_ARGUMENT;
-    return launch_grouped_gemm(X, off, W, B, E, R, K, N, dtype, epilogue, hint, Y, ws, ws_bytes, st(stream));
+    return launch_grouped_gemm(X, off, W, B, E, R, K, N, dtype, epilogue, hint, Y, ws, ws_bytes, st(stream), g);
 }
 
 int opmx_moe_column_parallel_linear(const void *X, const int64_t *expert_offset, const void *W, const void *B,
@@ -249,6 +285,20 @@ int opmx_moe_column_parallel_linear(const void *X, const int64_t *expert_offset,
 {
     return grouped_checked(X, expert_offset, W, B, E, R, K, N, dtype, epilogue, rows_per_expert_hint, Y,
                            workspace, workspace_bytes, stream);
+}
+
+int opmx_moe_column_parallel_linear_indexed(const void *X, int64_t X_rows, const int32_t *row_index,
+                                            const int64_t *expert_offset, const void *W, const void *B, int E,
+                                            int64_t R, int64_t K, int64_t N, int dtype, int epilogue,
+                                            int64_t rows_per_expert_hint, void *Y, void *workspace,
+                                            size_t workspace_bytes, void *stream)
+{
+    if (X_rows < 0 || (R > 0 && (X_rows == 0 || !row_index))) return OPMX_ERR_BAD_ARGUMENT;
+    RowGather g;
+    g.index = row_index;
+    g.x_rows = X_rows;
+    return grouped_checked(X, expert_offset, W, B, E, R, K, N, dtype, epilogue, rows_per_expert_hint, Y, workspace,
+                           workspace_bytes, stream, g);
 }
 
 int opmx_moe_row_parallel_linear(const void *X, const int64_t *expert_offset, const void *W, const void *B,

@@ -117,24 +117,23 @@ int cu_count();
 // Host launchers (one per translation unit); all return an opmx_status.
 int launch_linear(const void *X, const void *W, const void *B, int64_t T, int64_t K, int64_t N,
                   int dtype, void *Y, hipStream_t s);
+// Xp == nullptr: routing only (no row copy); row_token (may be nullptr) receives, for every row of the
+// permuted order, the token whose copy it is.
 int launch_moe_select(const void *X, const void *scores, int64_t T, int64_t H, int E, int k, int dtype,
                       void *Xp, void *w, int64_t *inv, int64_t *off, int32_t *ids, void *ws,
-                      hipStream_t s);
+                      hipStream_t s, int32_t *row_token = nullptr);
 size_t moe_select_workspace_bytes(int64_t T, int E, int k);
 int launch_moe_select_static(const void *X, const void *scores, int64_t T, int64_t H, int E, int k, int dtype,
                              void *Xp, void *w, int64_t *inv, int64_t *off, int32_t *ids, hipStream_t s);
 int launch_moe_route_select(const void *X, const void *Wg, const void *Bg, int64_t T, int64_t H, int E, int k,
                             int dtype, void *scores, void *Xp, void *w, int64_t *inv, int64_t *off, int32_t *ids,
-                            void *ws, hipStream_t s);
+                            void *ws, hipStream_t s, int32_t *row_token = nullptr);
 int launch_swiglu(const void *X, int64_t R, int64_t D, float beta, int dtype, void *Y, hipStream_t s);
 int launch_silu(const void *X, const void *gate, int64_t n, int dtype, void *Y, hipStream_t s);
 int launch_rms_norm(const void *X, const void *Wt, const void *Skip, int64_t T, int64_t H, float eps, int dtype,
                     void *Y, void *SkipOut, hipStream_t s);
 int launch_moe_reduce(const void *Y, const void *w, const int64_t *inv, int64_t T, int k, int64_t N,
                       int dtype, void *out, hipStream_t s);
-int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const void *B, int E,
-                        int64_t R, int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint,
-                        void *Y, void *ws, size_t ws_bytes, hipStream_t s);
 size_t grouped_gemm_workspace_bytes(int E, int64_t R, int64_t K, int64_t N, int dtype);
 
 }  // namespace opmx

@@ -64,6 +64,21 @@ template <> struct Mfma<bf16> {
     }
 };
 
+// Rows of a grouped GEMM's X operand taken through an index instead of in place: GEMM row r is
+// X[index[r], :] and X has x_rows rows (index == nullptr: row r is X[r, :]).  This is how the
+// gate/up GEMM reads the tokens of MoeSelect's permuted order without X_expand_permute
+// (MoeSelect.py:45-47) ever being written: index[r] = perm[r] / k.
+struct RowGather {
+    const int32_t *index = nullptr;
+    int64_t x_rows = 0;
+};
+// The row of X that GEMM row r reads, clamped into X (a corrupt index cannot leave the tensor).
+__device__ __forceinline__ int64_t gathered_row(const int32_t *__restrict__ index, int64_t x_rows, int64_t r)
+{
+    const int64_t t = index[r];
+    return t < 0 ? 0 : (t >= x_rows ? x_rows - 1 : t);
+}
+
 // One unit of grouped-GEMM work: `rows` rows starting at `row0`, all of expert `e`.
 struct MTile {
     int e;
@@ -171,17 +186,20 @@ __device__ __forceinline__ void zero_unowned_rows(T *__restrict__ Y, int64_t R, 
 }
 
 int launch_gemm_generic(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
-                        int64_t K, int64_t N, int dtype, int epilogue, void *Y, hipStream_t s);
+                        int64_t K, int64_t N, int dtype, int epilogue, void *Y, hipStream_t s, RowGather g = {});
 // variant: 0 = 256x256 direct-to-LDS kernel, 1 = 256x256 register-staged (8 waves),
 // 2 = 128x128 register-staged (4 waves).  off == nullptr: dense GEMM (one expert owns [0, R)).
 // ws / ws_bytes: optional scratch memory of gemm_tiled_workspace_bytes() bytes (variant 0 then
 // balances the last rounds of tiles over all CUs); nullptr / 0 is always accepted.
 int launch_gemm_tiled(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
                       int64_t K, int64_t N, int dtype, int epilogue, int variant, void *Y, void *ws,
-                      size_t ws_bytes, hipStream_t s);
+                      size_t ws_bytes, hipStream_t s, RowGather g = {});
 size_t gemm_tiled_workspace_bytes();
+int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const void *B, int E,
+                        int64_t R, int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint,
+                        void *Y, void *ws, size_t ws_bytes, hipStream_t s, RowGather g = {});
 int launch_gemm_stream(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
                        int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint, int variant, void *Y,
-                       hipStream_t s);
+                       hipStream_t s, RowGather g = {});
 
 }  // namespace opmx

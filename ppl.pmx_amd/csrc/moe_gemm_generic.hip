@@ -15,7 +15,8 @@ template <typename T, bool SWIGLU>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const T *__restrict__ X, const int64_t *__restrict__ off,
                                                            const T *__restrict__ W, const T *__restrict__ Bias,
                                                            int E, int64_t R, int64_t K, int64_t N,
-                                                           T *__restrict__ Y)
+                                                           T *__restrict__ Y, const int32_t *__restrict__ rt,
+                                                           int64_t xrows)
 {
     __shared__ float As[GK][GB + 4];
     __shared__ float Bs[SWIGLU ? 2 : 1][GK][GB + 4];
@@ -41,7 +42,9 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T *__restrict__
             const int q = threadIdx.x + 256 * i;
             const int row = q / GK, kk = q % GK;
             const bool kin = k0 + kk < K;
-            As[kk][row] = (row < mt.rows && kin) ? to_f32(X[(mt.row0 + row) * K + k0 + kk]) : 0.0f;
+            // the X row of tile row `row`: in place, or through the row index (RowGather)
+            const int64_t xr = (rt && row < mt.rows) ? gathered_row(rt, xrows, mt.row0 + row) : mt.row0 + row;
+            As[kk][row] = (row < mt.rows && kin) ? to_f32(X[xr * K + k0 + kk]) : 0.0f;
 #pragma unroll
             for (int h = 0; h < (SWIGLU ? 2 : 1); ++h) {
                 const int64_t n = n0 + row;
@@ -89,16 +92,16 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T *__restrict__
 
 template <typename T>
 int generic_impl(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
-                 int64_t N, int epilogue, void *Y, hipStream_t s)
+                 int64_t N, int epilogue, void *Y, hipStream_t s, RowGather g)
 {
     const int64_t ncols = epilogue == OPMX_EPILOGUE_SWIGLU ? N / 2 : N;
     dim3 grid(static_cast<unsigned>(ceil_div(ncols, GB)), static_cast<unsigned>(max_mtiles(R, E, GB)));
     if (epilogue == OPMX_EPILOGUE_SWIGLU)
         gemm_generic_kernel<T, true><<<grid, 256, 0, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
-                                                          static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y));
+                                                          static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), g.index, g.x_rows);
     else
         gemm_generic_kernel<T, false><<<grid, 256, 0, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
-                                                           static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y));
+                                                           static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), g.index, g.x_rows);
     OPMX_LAUNCH_CHECK();
     return OPMX_OK;
 }
@@ -106,12 +109,12 @@ int generic_impl(const void *X, const int64_t *off, const void *W, const void *B
 }  // namespace
 
 int launch_gemm_generic(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
-                        int64_t K, int64_t N, int dtype, int epilogue, void *Y, hipStream_t s)
+                        int64_t K, int64_t N, int dtype, int epilogue, void *Y, hipStream_t s, RowGather g)
 {
     switch (dtype) {
-        case OPMX_DTYPE_F32: return generic_impl<float>(X, off, W, B, E, R, K, N, epilogue, Y, s);
-        case OPMX_DTYPE_F16: return generic_impl<f16>(X, off, W, B, E, R, K, N, epilogue, Y, s);
-        case OPMX_DTYPE_BF16: return generic_impl<bf16>(X, off, W, B, E, R, K, N, epilogue, Y, s);
+        case OPMX_DTYPE_F32: return generic_impl<float>(X, off, W, B, E, R, K, N, epilogue, Y, s, g);
+        case OPMX_DTYPE_F16: return generic_impl<f16>(X, off, W, B, E, R, K, N, epilogue, Y, s, g);
+        case OPMX_DTYPE_BF16: return generic_impl<bf16>(X, off, W, B, E, R, K, N, epilogue, Y, s, g);
     }
     return OPMX_ERR_UNSUPPORTED;
 }

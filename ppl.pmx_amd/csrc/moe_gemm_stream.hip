@@ -38,7 +38,8 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
                                                                const int64_t *__restrict__ off,
                                                                const T *__restrict__ W,
                                                                const T *__restrict__ Bias, int E, int64_t R,
-                                                               int64_t K, int64_t N, T *__restrict__ Y)
+                                                               int64_t K, int64_t N, T *__restrict__ Y,
+                                                               const int32_t *__restrict__ rt, int64_t xrows)
 {
     // row groups per wave: SwiGLU pairs gate rows with up rows; PAIR gives a wave two adjacent
     // groups, so that a block shares its X chunk among twice the weight rows (tall row tiles,
@@ -77,7 +78,8 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
     // Rows past N are clamped to row N-1 (their results are masked at the store).
     const int64_t nbase = static_cast<int64_t>(blockIdx.x) * SROWS + (SGW ? (wave >> 1) * 16 : wave * WROWS);
     const char *wb = reinterpret_cast<const char *>(W + static_cast<int64_t>(mt.e) * N * K);
-    const char *xb = reinterpret_cast<const char *>(X + mt.row0 * K);
+    // X rows of this tile: in place from row0 on, or through the row index (RowGather; x_rows * K * 2 < 2^32)
+    const char *xb = reinterpret_cast<const char *>(rt ? X : X + mt.row0 * K);
     const int wl_row = lane / (64 / RPL);               // row inside one wave load
     const int wl_k = (lane % (64 / RPL)) * 8;           // k offset inside the chunk
     uint32_t wrow[NG][NLW];                             // byte offset of the row start
@@ -98,7 +100,7 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
     for (int i = 0; i < NLX; ++i) {
         const int q = tid + SW * 64 * i, row = q / CPR, c = q % CPR;
         const int r = row < mt.rows ? row : mt.rows - 1;
-        xrow[i] = static_cast<uint32_t>(r * K * 2);
+        xrow[i] = static_cast<uint32_t>((rt ? gathered_row(rt, xrows, mt.row0 + r) : r) * K * 2);
         xdst[i] = row * RS + c * 16;
         xk[i] = c * 8;
     }
@@ -230,7 +232,7 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
 
 template <typename T, int MT, int KC, int DEPTH, bool NT, int SW, bool SG, bool PAIR = false, bool SGW = false>
 int stream_launch_sw(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
-                     int64_t N, void *Y, hipStream_t s)
+                     int64_t N, void *Y, hipStream_t s, RowGather g)
 {
     constexpr int SROWS = SGW ? 16 * SW / 2 : (PAIR ? 32 : 16) * SW;
     constexpr int RS = KC * 2 + 16;
@@ -242,25 +244,25 @@ int stream_launch_sw(const void *X, const int64_t *off, const void *W, const voi
     dim3 grid(static_cast<unsigned>(ceil_div((SG || SGW) ? N / 2 : N, SROWS)),
               static_cast<unsigned>(max_mtiles(R, E, 16 * MT)));
     kern<<<grid, SW * 64, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
-                                     static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y));
+                                     static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), g.index, g.x_rows);
     OPMX_LAUNCH_CHECK();
     return OPMX_OK;
 }
 
 template <typename T, int MT, int KC, int DEPTH, bool NT, bool SG = false>
 int stream_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
-                  int64_t N, void *Y, hipStream_t s)
+                  int64_t N, void *Y, hipStream_t s, RowGather g)
 {
     // at most min(R, E) experts are active: with 64-column blocks that is this many work items
     const int64_t items = ceil_div(SG ? N / 2 : N, 64) * (R < E ? R : E);
     if (MT <= 2 && items < 512)
-        return stream_launch_sw<T, MT, KC, DEPTH, NT, 1, SG>(X, off, W, B, E, R, K, N, Y, s);
+        return stream_launch_sw<T, MT, KC, DEPTH, NT, 1, SG>(X, off, W, B, E, R, K, N, Y, s, g);
     // Tall row tiles: the X chunk a block stages is as large as its weight chunk, so every wave takes
     // two groups of weight rows and the block shares X among 128 of them (Mixtral gate/up at
     // T = 128: 357 -> 337 us, 64-row tiles; T = 256, 128-row tiles: 497 -> 374 us).
     if constexpr (MT >= 4 && !SG)
-        return stream_launch_sw<T, MT, KC, DEPTH, NT, 4, SG, true>(X, off, W, B, E, R, K, N, Y, s);
-    return stream_launch_sw<T, MT, KC, DEPTH, NT, 4, SG>(X, off, W, B, E, R, K, N, Y, s);
+        return stream_launch_sw<T, MT, KC, DEPTH, NT, 4, SG, true>(X, off, W, B, E, R, K, N, Y, s, g);
+    return stream_launch_sw<T, MT, KC, DEPTH, NT, 4, SG>(X, off, W, B, E, R, K, N, Y, s, g);
 }
 
 // Row-tile height MT*16 from the rows-per-expert bound m; K-chunk width per height
@@ -269,7 +271,7 @@ int stream_launch(const void *X, const int64_t *off, const void *W, const void *
 // instance only serves single-token calls.
 template <typename T, int KC1, int KC2, int KC4, int KC8, int DEPTH, bool NT>
 int stream_pick_mt(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
-                   int64_t N, int64_t m, void *Y, hipStream_t s)
+                   int64_t N, int64_t m, void *Y, hipStream_t s, RowGather g)
 {
     // A short K (fewer than 16 chunks of 256) is walked in chunks of 128: a block then lives for a
     // few chunks only, and the narrower chunks halve its LDS footprint, so that twice as many
@@ -278,53 +280,53 @@ int stream_pick_mt(const void *X, const int64_t *off, const void *W, const void 
     constexpr int KC1S = KC1 > 128 ? 128 : KC1, KC2S = KC2 > 128 ? 128 : KC2, KC4S = KC4 > 64 ? 64 : KC4;
     const bool short_k = K < 16 * 256;
     if (m <= 2)
-        return short_k ? stream_launch<T, 1, KC1S, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s)
-                       : stream_launch<T, 1, KC1, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
+        return short_k ? stream_launch<T, 1, KC1S, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s, g)
+                       : stream_launch<T, 1, KC1, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s, g);
     if (m <= 32)
-        return short_k ? stream_launch<T, 2, KC2S, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s)
-                       : stream_launch<T, 2, KC2, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
+        return short_k ? stream_launch<T, 2, KC2S, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s, g)
+                       : stream_launch<T, 2, KC2, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s, g);
     // 64-row tiles: 64-wide chunks up to K = 8192 (Mixtral gate/up, K = 4096, at T = 128: 337 -> 322 us),
     // 128-wide beyond (down projection, K = 14336: 162 us against 175 with 64-wide chunks)
     if (m <= 64)
-        return K <= 8192 ? stream_launch<T, 4, KC4S, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s)
-                         : stream_launch<T, 4, KC4, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
-    return stream_launch<T, 8, KC8, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s);
+        return K <= 8192 ? stream_launch<T, 4, KC4S, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s, g)
+                         : stream_launch<T, 4, KC4, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s, g);
+    return stream_launch<T, 8, KC8, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s, g);
 }
 
 // SwiGLU epilogue: a wave streams twice the rows, so the K chunks are half as wide.
 template <typename T>
 int stream_swiglu_impl(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
-                       int64_t N, int64_t rows_hint, void *Y, hipStream_t s)
+                       int64_t N, int64_t rows_hint, void *Y, hipStream_t s, RowGather g)
 {
     const int64_t m = rows_hint > 0 ? rows_hint : R;
     if (m <= 2)      // short K: narrower chunks, as in stream_pick_mt
-        return K < 16 * 256 ? stream_launch<T, 1, 128, 2, true, true>(X, off, W, B, E, R, K, N, Y, s)
-                            : stream_launch<T, 1, 256, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);
+        return K < 16 * 256 ? stream_launch<T, 1, 128, 2, true, true>(X, off, W, B, E, R, K, N, Y, s, g)
+                            : stream_launch<T, 1, 256, 2, true, true>(X, off, W, B, E, R, K, N, Y, s, g);
     if (m <= 32) {
         // long K: SwiGLU by wave pairs, which keeps the plain form's 256-wide chunks and LDS footprint
         // (a wave with two row groups needs twice the strip: chunks half as wide, or half the waves
         // per CU).  Decode T=32, layer: 0.452 ms with two groups per wave, 0.442 by pairs (unfused 0.440).
         const int64_t items = ceil_div(N / 2, 64) * (R < E ? R : E);
         if (K >= 16 * 256 && items >= 512)
-            return stream_launch_sw<T, 2, 256, 2, true, 4, false, false, true>(X, off, W, B, E, R, K, N, Y, s);
-        return stream_launch<T, 2, 128, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);
+            return stream_launch_sw<T, 2, 256, 2, true, 4, false, false, true>(X, off, W, B, E, R, K, N, Y, s, g);
+        return stream_launch<T, 2, 128, 2, true, true>(X, off, W, B, E, R, K, N, Y, s, g);
     }
-    if (m <= 64) return stream_launch<T, 4, 64, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);
-    return stream_launch<T, 8, 64, 2, true, true>(X, off, W, B, E, R, K, N, Y, s);
+    if (m <= 64) return stream_launch<T, 4, 64, 2, true, true>(X, off, W, B, E, R, K, N, Y, s, g);
+    return stream_launch<T, 8, 64, 2, true, true>(X, off, W, B, E, R, K, N, Y, s, g);
 }
 
 template <typename T>
 int stream_impl(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
-                int64_t N, int64_t rows_hint, int variant, void *Y, hipStream_t s)
+                int64_t N, int64_t rows_hint, int variant, void *Y, hipStream_t s, RowGather g)
 {
     const int64_t m = rows_hint > 0 ? rows_hint : R;
     switch (variant) {   // tuning knob; every variant computes the same thing
-        case 1: return stream_pick_mt<T, 256, 256, 128, 128, 1, false>(X, off, W, B, E, R, K, N, m, Y, s);
-        case 2: return stream_pick_mt<T, 512, 512, 256, 128, 1, true>(X, off, W, B, E, R, K, N, m, Y, s);
-        case 3: return stream_pick_mt<T, 256, 256, 128, 64, 2, false>(X, off, W, B, E, R, K, N, m, Y, s);
-        case 4: return stream_pick_mt<T, 256, 128, 64, 64, 2, true>(X, off, W, B, E, R, K, N, m, Y, s);
-        case 5: return stream_pick_mt<T, 256, 256, 128, 128, 2, true>(X, off, W, B, E, R, K, N, m, Y, s);
-        default: return stream_pick_mt<T, 256, 256, 128, 64, 2, true>(X, off, W, B, E, R, K, N, m, Y, s);
+        case 1: return stream_pick_mt<T, 256, 256, 128, 128, 1, false>(X, off, W, B, E, R, K, N, m, Y, s, g);
+        case 2: return stream_pick_mt<T, 512, 512, 256, 128, 1, true>(X, off, W, B, E, R, K, N, m, Y, s, g);
+        case 3: return stream_pick_mt<T, 256, 256, 128, 64, 2, false>(X, off, W, B, E, R, K, N, m, Y, s, g);
+        case 4: return stream_pick_mt<T, 256, 128, 64, 64, 2, true>(X, off, W, B, E, R, K, N, m, Y, s, g);
+        case 5: return stream_pick_mt<T, 256, 256, 128, 128, 2, true>(X, off, W, B, E, R, K, N, m, Y, s, g);
+        default: return stream_pick_mt<T, 256, 256, 128, 64, 2, true>(X, off, W, B, E, R, K, N, m, Y, s, g);
     }
 }
 
@@ -333,16 +335,16 @@ int stream_impl(const void *X, const int64_t *off, const void *W, const void *B,
 // Requires: dtype f16/bf16, K % 8 == 0, 16-byte aligned X and W.
 int launch_gemm_stream(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
                        int64_t K, int64_t N, int dtype, int epilogue, int64_t rows_hint, int variant, void *Y,
-                       hipStream_t s)
+                       hipStream_t s, RowGather g)
 {
     if (epilogue == OPMX_EPILOGUE_SWIGLU) {
-        if (dtype == OPMX_DTYPE_F16) return stream_swiglu_impl<f16>(X, off, W, B, E, R, K, N, rows_hint, Y, s);
-        if (dtype == OPMX_DTYPE_BF16) return stream_swiglu_impl<bf16>(X, off, W, B, E, R, K, N, rows_hint, Y, s);
+        if (dtype == OPMX_DTYPE_F16) return stream_swiglu_impl<f16>(X, off, W, B, E, R, K, N, rows_hint, Y, s, g);
+        if (dtype == OPMX_DTYPE_BF16) return stream_swiglu_impl<bf16>(X, off, W, B, E, R, K, N, rows_hint, Y, s, g);
         return OPMX_ERR_UNSUPPORTED;
     }
     switch (dtype) {
-        case OPMX_DTYPE_F16: return stream_impl<f16>(X, off, W, B, E, R, K, N, rows_hint, variant, Y, s);
-        case OPMX_DTYPE_BF16: return stream_impl<bf16>(X, off, W, B, E, R, K, N, rows_hint, variant, Y, s);
+        case OPMX_DTYPE_F16: return stream_impl<f16>(X, off, W, B, E, R, K, N, rows_hint, variant, Y, s, g);
+        case OPMX_DTYPE_BF16: return stream_impl<bf16>(X, off, W, B, E, R, K, N, rows_hint, variant, Y, s, g);
     }
     return OPMX_ERR_UNSUPPORTED;
 }

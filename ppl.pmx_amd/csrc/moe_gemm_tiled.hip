@@ -451,7 +451,8 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
                                                                   const T *__restrict__ W,
                                                                   const T *__restrict__ Bias, int E, int64_t R,
                                                                   int64_t K, int64_t N, T *__restrict__ Y,
-                                                                  int ntiles_n, int gnx)
+                                                                  int ntiles_n, int gnx,
+                                                                  const int32_t *__restrict__ rt, int64_t xrows)
 {
     constexpr int NT = WM * WN * 64;
     constexpr int WTM = BM / WM, WTN = BN / WN;          // wave tile: WTM X-rows x WTN W-rows
@@ -482,7 +483,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     const int64_t n0 = static_cast<int64_t>(tile_n) * BNO;
-    const T *Xt = X + mt.row0 * K;
+    const T *Xt = rt ? X : X + mt.row0 * K;      // with a row index (RowGather) offsets count from X itself
     const T *We = W + static_cast<int64_t>(mt.e) * N * K;
 
     // Staging: load q of a thread covers tile row tid/8 + RSTEP*q, 16-byte chunk tid%8.
@@ -495,7 +496,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tiled_kernel(const T *__rest
     for (int i = 0; i < LA; ++i) {
         const int row = srow + RSTEP * i;
         const int r = row < mt.rows ? row : mt.rows - 1;
-        a_src[i] = static_cast<uint32_t>((r * K + sc * 8) * 2);
+        a_src[i] = static_cast<uint32_t>(((rt ? gathered_row(rt, xrows, mt.row0 + r) : r) * K + sc * 8) * 2);
     }
 #pragma unroll
     for (int i = 0; i < LB; ++i) {
@@ -718,6 +719,8 @@ __device__ __forceinline__ void load_to_lds_16(__amdgpu_buffer_rsrc_t r, char *l
     __builtin_amdgcn_raw_ptr_buffer_load_lds(r, OPMX_LPTR(lds), 16, voff, soff, 0, 0);
 }
 
+constexpr uint32_t kPastEveryX = 0x80000000u;   // a byte offset no gathered X reaches (x_descriptor)
+
 // This lane's share of the sixteen 1 KiB wave loads per operand and k-tile: load i of wave w
 // fetches tile rows 8*(w*L+i) .. +7, lane l the 16-byte chunk of row 8*(w*L+i) + l/8 that
 // belongs in LDS slot l%8 of that row (slots are XOR-swizzled by row).  Results are byte offsets
@@ -729,15 +732,24 @@ __device__ __forceinline__ void load_to_lds_16(__amdgpu_buffer_rsrc_t r, char *l
 // MFMA kernels against a power limit.  With SWIGLU a wave's WTN W-rows are WTN/2 gate rows
 // followed by the WTN/2 up rows of the same output columns.
 template <int LA, int LB, int WTN, bool SWIGLU>
-__device__ __forceinline__ void tile_sources(int /*rows*/, int64_t n0, int64_t K, int64_t N, int64_t ncols, int wave,
-                                             int lane, uint32_t (&a_src)[LA], uint32_t (&b_src)[LB])
+__device__ __forceinline__ void tile_sources(int rows, bool gather, int tokv, int64_t n0, int64_t K, int64_t N,
+                                             int64_t ncols, int wave, int lane, uint32_t (&a_src)[LA],
+                                             uint32_t (&b_src)[LB])
 {
     const int lrow8 = lane >> 3, slot = lane & 7;
 #pragma unroll
     for (int i = 0; i < LA; ++i) {
         const int row = (wave * LA + i) * 8 + lrow8;
         const int c = slot ^ ((row >> 1) & 7);
-        a_src[i] = static_cast<uint32_t>((row * K + c * 8) * 2);
+        if (!gather) {
+            a_src[i] = static_cast<uint32_t>((row * K + c * 8) * 2);
+        } else {
+            // Through the row index (RowGather): offsets count from X itself.  Lane l of the wave
+            // holds the index of the wave's l-th row (wave_row_index); each lane fetches the one of
+            // its row by a cross-lane read.  Rows the tile lacks get an offset past every X.
+            const int tok = __shfl(tokv, i * 8 + lrow8, 64);
+            a_src[i] = row < rows ? static_cast<uint32_t>((static_cast<int64_t>(tok) * K + c * 8) * 2) : kPastEveryX;
+        }
     }
 #pragma unroll
     for (int i = 0; i < LB; ++i) {
@@ -756,11 +768,26 @@ __device__ __forceinline__ void tile_sources(int /*rows*/, int64_t n0, int64_t K
     }
 }
 
-// Descriptor of a tile's X rows: `rows` rows of K elements from row `row0` on, and nothing behind
-// them (loads of the rows a ragged tile lacks return zeros, see tile_sources).
-template <typename T>
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t x_descriptor(const T *X, int64_t row0, int rows, int64_t K)
+// Row index (RowGather) of the l-th X row that wave `wave` loads for the tile starting at row0
+// (a wave loads RW = BM / 4 consecutive tile rows), in lane l; 0 without an index.  One load per
+// lane, issued well ahead of tile_sources, which reads it across lanes.
+template <int RW>
+__device__ __forceinline__ int wave_row_index(const int32_t *__restrict__ rt, int64_t row0, int64_t R, int wave, int lane)
 {
+    if (rt == nullptr) return 0;
+    const int64_t r = row0 + wave * RW + (lane < RW ? lane : RW - 1);
+    return rt[r < R ? r : R - 1];
+}
+
+// Descriptor of a tile's X rows: `rows` rows of K elements from row `row0` on, and nothing behind
+// them (loads of the rows a ragged tile lacks return zeros, see tile_sources).  With a row index
+// (RowGather) it covers all xrows rows of X (xrows * K * 2 < 2^31) and tile_sources gives the
+// lacking rows the offset kPastEveryX.
+template <typename T>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t x_descriptor(const T *X, int64_t row0, int rows, int64_t K,
+                                                               const int32_t *rt, int64_t xrows)
+{
+    if (rt) return bounded_descriptor(X, static_cast<uint32_t>(xrows * K * 2));
     return bounded_descriptor(X + row0 * K, static_cast<uint32_t>(rows * K * 2));
 }
 
@@ -839,7 +866,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
                                                                const T *__restrict__ Bias, int E, int64_t R,
                                                                int64_t K, int64_t N, T *__restrict__ Y,
                                                                int ntiles_n, int gnx, int sk_wgs, int sk_cost,
-                                                               float *__restrict__ sk_part, int *__restrict__ sk_count)
+                                                               float *__restrict__ sk_part, int *__restrict__ sk_count,
+                                                               const int32_t *__restrict__ rt, int64_t xrows)
 {
     constexpr int NW = 4, WM = BM / 128, WN = NW / WM;                 // 256 x 256: 2 x 2 waves, 128 x 256: 1 x 4
     constexpr int WTM = BM / WM, WTN = BN / WN, TMS = WTM / 16, TNS = WTN / 16, HM = TMS / 2;
@@ -897,11 +925,12 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
     const int64_t n0 = static_cast<int64_t>(tile_n) * BNO;
-    const __amdgpu_buffer_rsrc_t rx = x_descriptor(X, mt.row0, mt.rows, K);
+    const __amdgpu_buffer_rsrc_t rx = x_descriptor(X, mt.row0, mt.rows, K, rt, xrows);
     const __amdgpu_buffer_rsrc_t rw = raw_descriptor(W + static_cast<int64_t>(mt.e) * N * K);
 
     uint32_t a_src[LA], b_src[LB];     // byte offsets from the tile's X / W base at k = 0
-    tile_sources<LA, LB, WTN, SWIGLU>(mt.rows, n0, K, N, ncols, wave, lane, a_src, b_src);
+    tile_sources<LA, LB, WTN, SWIGLU>(mt.rows, rt != nullptr, wave_row_index<LA * 8>(rt, mt.row0, R, wave, lane), n0, K, N,
+                                      ncols, wave, lane, a_src, b_src);
     const int a_lds = wave * LA * 1024, b_lds = BM * ROWB + wave * LB * 1024;   // wave-uniform
 
     float4_t acc[TNS][TMS];
@@ -1181,7 +1210,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
                                                                        const T *__restrict__ W,
                                                                        const T *__restrict__ Bias, int E, int64_t R,
                                                                        int64_t K, int64_t N, T *__restrict__ Y,
-                                                                       int ntiles_n, int gnx, int sk_wgs, int sk_cost)
+                                                                       int ntiles_n, int gnx, int sk_wgs, int sk_cost,
+                                                                       const int32_t *__restrict__ rt, int64_t xrows)
 {
     constexpr int WM = 2, WN = 2, NW = 4;
     constexpr int WTM = BM / WM, WTN = BN / WN, TMS = WTM / 16, TNS = WTN / 16, HM = TMS / 2;
@@ -1223,10 +1253,11 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
     int cur_n;
     locate_any(id, gnx, mtiles, ntiles_n, off != nullptr, s_off, E, R, BM, cur, cur_n);
     if (cur.rows == 0) return;
-    __amdgpu_buffer_rsrc_t rx = x_descriptor(X, cur.row0, cur.rows, K);
+    __amdgpu_buffer_rsrc_t rx = x_descriptor(X, cur.row0, cur.rows, K, rt, xrows);
     __amdgpu_buffer_rsrc_t rw = raw_descriptor(W + static_cast<int64_t>(cur.e) * N * K);
     uint32_t a_src[LA], b_src[LB];
-    tile_sources<LA, LB, WTN, SWIGLU>(cur.rows, static_cast<int64_t>(cur_n) * BNO, K, N, ncols, wave, lane, a_src, b_src);
+    tile_sources<LA, LB, WTN, SWIGLU>(cur.rows, rt != nullptr, wave_row_index<LA * 8>(rt, cur.row0, R, wave, lane),
+                                      static_cast<int64_t>(cur_n) * BNO, K, N, ncols, wave, lane, a_src, b_src);
     const int a_lds = wave * LA * 1024, b_lds = BM * ROWB + wave * LB * 1024;
     char *stg = smem + 2 * STAGE + wave * STG;
 
@@ -1276,6 +1307,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
             if (has_next) nxt = t;
             else nxt_n = cur_n;
         }
+        // the next tile's row indices (RowGather), requested a whole tile ahead of their use
+        const int nxt_tok = wave_row_index<LA * 8>(rt, nxt.row0, R, wave, lane);
 
         // k-tile 0 overwrites the accumulators.  When k-tile 1 is known to have landed, the NS
         // stores of the previous tile and the 16 loads of this step may still be outstanding.
@@ -1283,9 +1316,10 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
         b ^= 1;
         for (int kt = 1; kt + 2 < nk; ++kt, b ^= 1) OPMX_ITERX(kt + 2, b, true, true, false, 16);
         // all loads of this tile are issued: retarget the load state, then stream on
-        rx = x_descriptor(X, nxt.row0, nxt.rows, K);
+        rx = x_descriptor(X, nxt.row0, nxt.rows, K, rt, xrows);
         rw = raw_descriptor(W + static_cast<int64_t>(nxt.e) * N * K);
-        tile_sources<LA, LB, WTN, SWIGLU>(nxt.rows, static_cast<int64_t>(nxt_n) * BNO, K, N, ncols, wave, lane, a_src, b_src);
+        tile_sources<LA, LB, WTN, SWIGLU>(nxt.rows, rt != nullptr, nxt_tok, static_cast<int64_t>(nxt_n) * BNO, K, N, ncols, wave,
+                                          lane, a_src, b_src);
         const int64_t nw0 = static_cast<int64_t>(cur_n) * BNO + wn * (SWIGLU ? WTN / 2 : WTN);   // first output column of this wave
         T bg[NOB][4], bu[NOB][4];          // bias of this lane's columns, requested ahead of the last loads
         if (BIAS) load_bias_regs<T, NOB, SWIGLU>(Bias + static_cast<int64_t>(cur.e) * N, ncols, nw0, lane, bg, bu);
@@ -1333,7 +1367,7 @@ __global__ void sk_clear_kernel(int *__restrict__ count, int n)
 
 template <typename T, int BM, int BN, int WM, int WN>
 int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
-                   int64_t N, int epilogue, void *Y, hipStream_t s)
+                   int64_t N, int epilogue, void *Y, hipStream_t s, RowGather g)
 {
     constexpr int smem = 2 * (BM + BN) * ROWB;
     const bool sw = epilogue == OPMX_EPILOGUE_SWIGLU;
@@ -1349,12 +1383,14 @@ int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B
         auto kern = gemm_tiled_kernel<T, BM, BN, WM, WN, true>;
         if (!ensure_dynamic_smem(reinterpret_cast<const void *>(kern), smem, attr_done[1])) return OPMX_ERR_LAUNCH;
         kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
-                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_n, gnx);
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_n, gnx, g.index,
+                                       g.x_rows);
     } else {
         auto kern = gemm_tiled_kernel<T, BM, BN, WM, WN, false>;
         if (!ensure_dynamic_smem(reinterpret_cast<const void *>(kern), smem, attr_done[0])) return OPMX_ERR_LAUNCH;
         kern<<<grid, block, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
-                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_n, gnx);
+                                       static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), ntiles_n, gnx, g.index,
+                                       g.x_rows);
     }
     OPMX_LAUNCH_CHECK();
     return OPMX_OK;
@@ -1372,7 +1408,7 @@ size_t sk_workspace_bytes(int cus)
 
 template <typename T, int BM, int BN>
 int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
-                      int64_t K, int64_t N, int epilogue, void *Y, void *ws, size_t ws_bytes, hipStream_t s)
+                      int64_t K, int64_t N, int epilogue, void *Y, void *ws, size_t ws_bytes, hipStream_t s, RowGather g)
 {
     static_assert(BM * BN <= kSkTile, "tail slot size");
     constexpr int smem = 2 * (BM + BN) * ROWB;
@@ -1428,7 +1464,7 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
         static std::atomic<uint64_t> attr_p[4];
         const bool hb = B != nullptr;
         using kernel_t = void (*)(const T *, const int64_t *, const T *, const T *, int, int64_t, int64_t, int64_t, T *, int,
-                                  int, int, int);
+                                  int, int, int, const int32_t *, int64_t);
         const kernel_t kp = sw ? (hb ? gemm_tiled_dlds_persist_kernel<T, BM, BN, true, true>
                                      : gemm_tiled_dlds_persist_kernel<T, BM, BN, true, false>)
                                : (hb ? gemm_tiled_dlds_persist_kernel<T, BM, BN, false, true>
@@ -1438,14 +1474,14 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
         // ids congruent mod 8 stay on one XCD as long as the grid is a multiple of 8
         const unsigned wgs = static_cast<unsigned>(dp_ids < cus ? dp_ids : cus);
         if (sk_wgs > 0) sk_clear_kernel<<<1, 256, 0, s>>>(sk_count, kSkCounters);
-        kp<<<wgs, block, smem_p, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n, gnx, sk_wgs, sk_cost);
+        kp<<<wgs, block, smem_p, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n, gnx, sk_wgs, sk_cost, g.index, g.x_rows);
         if (sk_wgs > 0) {
             if (sw)
                 gemm_tiled_dlds_kernel<T, BM, BN, true, true><<<sk_wgs, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
-                                                                                          gnx, sk_wgs, sk_cost, sk_part, sk_count);
+                                                                                          gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows);
             else
                 gemm_tiled_dlds_kernel<T, BM, BN, false, true><<<sk_wgs, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
-                                                                                           gnx, sk_wgs, sk_cost, sk_part, sk_count);
+                                                                                           gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows);
         }
         OPMX_LAUNCH_CHECK();
         return OPMX_OK;
@@ -1453,16 +1489,16 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
     if (sk_wgs > 0) sk_clear_kernel<<<1, 256, 0, s>>>(sk_count, kSkCounters);
     if (sw) {
         gemm_tiled_dlds_kernel<T, BM, BN, true, false><<<grid, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
-                                                                                 gnx, sk_wgs, sk_cost, sk_part, sk_count);
+                                                                                 gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows);
         if (sk_wgs > 0)
             gemm_tiled_dlds_kernel<T, BM, BN, true, true><<<sk_wgs, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
-                                                                                      gnx, sk_wgs, sk_cost, sk_part, sk_count);
+                                                                                      gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows);
     } else {
         gemm_tiled_dlds_kernel<T, BM, BN, false, false><<<grid, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
-                                                                                  gnx, sk_wgs, sk_cost, sk_part, sk_count);
+                                                                                  gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows);
         if (sk_wgs > 0)
             gemm_tiled_dlds_kernel<T, BM, BN, false, true><<<sk_wgs, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
-                                                                                       gnx, sk_wgs, sk_cost, sk_part, sk_count);
+                                                                                       gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows);
     }
     OPMX_LAUNCH_CHECK();
     return OPMX_OK;
@@ -1470,13 +1506,13 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
 
 template <typename T>
 int tiled_impl(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
-               int64_t N, int epilogue, int variant, void *Y, void *ws, size_t ws_bytes, hipStream_t s)
+               int64_t N, int epilogue, int variant, void *Y, void *ws, size_t ws_bytes, hipStream_t s, RowGather g)
 {
     switch (variant) {
-        case 1: return tiled_launch<T, 256, 256, 2, 4>(X, off, W, B, E, R, K, N, epilogue, Y, s);
-        case 2: return tiled_launch<T, 128, 128, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s);
-        case 3: return tiled_dlds_launch<T, 128, 256>(X, off, W, B, E, R, K, N, epilogue, Y, ws, ws_bytes, s);
-        default: return tiled_dlds_launch<T, 256, 256>(X, off, W, B, E, R, K, N, epilogue, Y, ws, ws_bytes, s);
+        case 1: return tiled_launch<T, 256, 256, 2, 4>(X, off, W, B, E, R, K, N, epilogue, Y, s, g);
+        case 2: return tiled_launch<T, 128, 128, 2, 2>(X, off, W, B, E, R, K, N, epilogue, Y, s, g);
+        case 3: return tiled_dlds_launch<T, 128, 256>(X, off, W, B, E, R, K, N, epilogue, Y, ws, ws_bytes, s, g);
+        default: return tiled_dlds_launch<T, 256, 256>(X, off, W, B, E, R, K, N, epilogue, Y, ws, ws_bytes, s, g);
     }
 }
 
@@ -1487,11 +1523,13 @@ int tiled_impl(const void *X, const int64_t *off, const void *W, const void *B, 
 // variant balances the last rounds of tiles over all CUs.
 int launch_gemm_tiled(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
                       int64_t K, int64_t N, int dtype, int epilogue, int variant, void *Y, void *ws,
-                      size_t ws_bytes, hipStream_t s)
+                      size_t ws_bytes, hipStream_t s, RowGather g)
 {
+    // offsets into a gathered X are 32 bits wide and kPastEveryX must lie behind it
+    if (g.index != nullptr && g.x_rows * K * 2 >= (int64_t{1} << 31)) return OPMX_ERR_UNSUPPORTED;
     switch (dtype) {
-        case OPMX_DTYPE_F16: return tiled_impl<f16>(X, off, W, B, E, R, K, N, epilogue, variant, Y, ws, ws_bytes, s);
-        case OPMX_DTYPE_BF16: return tiled_impl<bf16>(X, off, W, B, E, R, K, N, epilogue, variant, Y, ws, ws_bytes, s);
+        case OPMX_DTYPE_F16: return tiled_impl<f16>(X, off, W, B, E, R, K, N, epilogue, variant, Y, ws, ws_bytes, s, g);
+        case OPMX_DTYPE_BF16: return tiled_impl<bf16>(X, off, W, B, E, R, K, N, epilogue, variant, Y, ws, ws_bytes, s, g);
     }
     return OPMX_ERR_UNSUPPORTED;
 }

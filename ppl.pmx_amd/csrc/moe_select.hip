@@ -264,7 +264,8 @@ __global__ __launch_bounds__(1024) void select_scan_kernel(int32_t *__restrict__
 __global__ __launch_bounds__(kChunk) void select_rank_kernel(const int32_t *__restrict__ ids,
                                                              const int32_t *__restrict__ base,
                                                              const int64_t *__restrict__ off, int64_t Ttok,
-                                                             int E, int k, int64_t *__restrict__ inv)
+                                                             int E, int k, int64_t *__restrict__ inv,
+                                                             int32_t *__restrict__ row_token)
 {
     __shared__ uint32_t bits[OPMX_MOE_MAX_EXPERTS * kWords];
     __shared__ int wordpre[OPMX_MOE_MAX_EXPERTS * kWords];
@@ -281,8 +282,9 @@ __global__ __launch_bounds__(kChunk) void select_rank_kernel(const int32_t *__re
     if (t < Ttok)
         for (int s = 0; s < k; ++s) {
             int e = ids[t * k + s];
-            inv[t * k + s] = off[e] + base[static_cast<int64_t>(blockIdx.x) * E + e] +
-                             rank_in_chunk(bits, wordpre, e, tl);
+            const int64_t pos = off[e] + base[static_cast<int64_t>(blockIdx.x) * E + e] + rank_in_chunk(bits, wordpre, e, tl);
+            inv[t * k + s] = pos;
+            if (row_token) row_token[pos] = static_cast<int32_t>(t);   // the token whose copy row `pos` is (perm[pos] / k)
         }
 }
 
@@ -388,7 +390,8 @@ __global__ __launch_bounds__(1024) void select_small_kernel(const T *__restrict_
                                                               int64_t *__restrict__ off,
                                                               int32_t *__restrict__ ids_out, bool vec,
                                                               const T *__restrict__ Wg, const T *__restrict__ Bg,
-                                                              T *__restrict__ scores_out)
+                                                              T *__restrict__ scores_out,
+                                                              int32_t *__restrict__ row_token)
 {
     __shared__ uint32_t bits[OPMX_MOE_MAX_EXPERTS * kWords];
     __shared__ int wordpre[OPMX_MOE_MAX_EXPERTS * kWords];
@@ -442,14 +445,16 @@ __global__ __launch_bounds__(1024) void select_small_kernel(const T *__restrict_
         int64_t pos = count[e] + rank_in_chunk(bits, wordpre, e, me);
         my_inv[threadIdx.x] = pos;
         inv[static_cast<int64_t>(me) * k + threadIdx.x] = pos;
+        if (row_token) row_token[pos] = me;
     }
+    if (Xp == nullptr) return;              // routing only: the caller reads X through row_token
     __syncthreads();
     expand_row(X, Xp, static_cast<int64_t>(me), H, k, my_inv, vec);
 }
 
 template <typename T>
 int select_impl(const void *X_, const void *scores_, int64_t Ttok, int64_t H, int E, int k, void *Xp_, void *w_,
-                int64_t *inv, int64_t *off, int32_t *ids, void *ws, hipStream_t s)
+                int64_t *inv, int64_t *off, int32_t *ids, void *ws, hipStream_t s, int32_t *row_token)
 {
     const T *X = static_cast<const T *>(X_);
     const T *scores = static_cast<const T *>(scores_);
@@ -474,7 +479,7 @@ int select_impl(const void *X_, const void *scores_, int64_t Ttok, int64_t H, in
         // wide lane groups (many experts) route few tokens per wave: use a big block
         const unsigned threads = G >= 32 ? 1024 : kChunk;
         select_small_kernel<T, false><<<static_cast<unsigned>(Ttok), threads, 0, s>>>(
-            X, scores, static_cast<int>(Ttok), H, E, k, G, vpl, Xp, w, inv, off, ids, vec, nullptr, nullptr, nullptr);
+            X, scores, static_cast<int>(Ttok), H, E, k, G, vpl, Xp, w, inv, off, ids, vec, nullptr, nullptr, nullptr, row_token);
         OPMX_LAUNCH_CHECK();
         return OPMX_OK;
     }
@@ -487,7 +492,7 @@ int select_impl(const void *X_, const void *scores_, int64_t Ttok, int64_t H, in
                                                                                                    vpl, w, idbuf);
         OPMX_LAUNCH_CHECK();
         select_small_kernel<T, false><<<static_cast<unsigned>(Ttok), kChunk, 0, s>>>(
-            X, nullptr, static_cast<int>(Ttok), H, E, k, G, vpl, Xp, w, inv, off, idbuf, vec, nullptr, nullptr, nullptr);
+            X, nullptr, static_cast<int>(Ttok), H, E, k, G, vpl, Xp, w, inv, off, idbuf, vec, nullptr, nullptr, nullptr, row_token);
         OPMX_LAUNCH_CHECK();
         return OPMX_OK;
     }
@@ -498,26 +503,29 @@ int select_impl(const void *X_, const void *scores_, int64_t Ttok, int64_t H, in
     OPMX_LAUNCH_CHECK();
     select_scan_kernel<<<1, E > 16 ? 1024 : 256, 0, s>>>(hist, nchunks, E, R, off);
     OPMX_LAUNCH_CHECK();
-    select_rank_kernel<<<nchunks, kChunk, 0, s>>>(idbuf, hist, off, Ttok, E, k, inv);
+    select_rank_kernel<<<nchunks, kChunk, 0, s>>>(idbuf, hist, off, Ttok, E, k, inv, row_token);
     OPMX_LAUNCH_CHECK();
-    const unsigned grid = static_cast<unsigned>(Ttok < 65536 ? Ttok : 65536);
-    select_expand_kernel<T><<<grid, 256, 0, s>>>(X, Xp, inv, Ttok, H, k, vec);
-    OPMX_LAUNCH_CHECK();
+    if (Xp != nullptr) {                   // nullptr: routing only, the caller reads X through row_token
+        const unsigned grid = static_cast<unsigned>(Ttok < 65536 ? Ttok : 65536);
+        select_expand_kernel<T><<<grid, 256, 0, s>>>(X, Xp, inv, Ttok, H, k, vec);
+        OPMX_LAUNCH_CHECK();
+    }
     return OPMX_OK;
 }
 
 template <typename T>
 int route_select_fused(const void *X_, const void *Wg_, const void *Bg_, int64_t Ttok, int64_t H, int E, int k,
-                       void *scores_, void *Xp_, void *w_, int64_t *inv, int64_t *off, int32_t *ids, hipStream_t s)
+                       void *scores_, void *Xp_, void *w_, int64_t *inv, int64_t *off, int32_t *ids, hipStream_t s,
+                       int32_t *row_token)
 {
     const T *X = static_cast<const T *>(X_);
     T *Xp = static_cast<T *>(Xp_);
     int G = 8;
     while (G < E) G <<= 1;
-    const bool vec = (H * sizeof(T)) % 16 == 0 && aligned16(X) && aligned16(Xp);
+    const bool vec = (H * sizeof(T)) % 16 == 0 && aligned16(X) && aligned16(Xp);   // (unused without Xp)
     select_small_kernel<T, true><<<static_cast<unsigned>(Ttok), kFusedWaves * kWave, 0, s>>>(
         X, nullptr, static_cast<int>(Ttok), H, E, k, G, (E + G - 1) / G, Xp, static_cast<T *>(w_), inv, off, ids, vec,
-        static_cast<const T *>(Wg_), static_cast<const T *>(Bg_), static_cast<T *>(scores_));
+        static_cast<const T *>(Wg_), static_cast<const T *>(Bg_), static_cast<T *>(scores_), row_token);
     OPMX_LAUNCH_CHECK();
     return OPMX_OK;
 }
@@ -529,19 +537,19 @@ int route_select_fused(const void *X_, const void *Wg_, const void *Bg_, int64_t
 // otherwise the two operators one after the other.  `scores` [T,E] receives the logits either way.
 int launch_moe_route_select(const void *X, const void *Wg, const void *Bg, int64_t T, int64_t H, int E, int k,
                             int dtype, void *scores, void *Xp, void *w, int64_t *inv, int64_t *off, int32_t *ids,
-                            void *ws, hipStream_t s)
+                            void *ws, hipStream_t s, int32_t *row_token)
 {
     const bool lowp = dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16;
     static_assert(kFusedMaxTokens <= kFusedTokens, "one MFMA tile of tokens");
     if (lowp && T >= 1 && T <= kFusedMaxTokens && E <= kFusedExperts && H >= 32 && H % 32 == 0 && aligned16(X) &&
         aligned16(Wg)) {
         if (dtype == OPMX_DTYPE_F16)
-            return route_select_fused<f16>(X, Wg, Bg, T, H, E, k, scores, Xp, w, inv, off, ids, s);
-        return route_select_fused<bf16>(X, Wg, Bg, T, H, E, k, scores, Xp, w, inv, off, ids, s);
+            return route_select_fused<f16>(X, Wg, Bg, T, H, E, k, scores, Xp, w, inv, off, ids, s, row_token);
+        return route_select_fused<bf16>(X, Wg, Bg, T, H, E, k, scores, Xp, w, inv, off, ids, s, row_token);
     }
     const int rc = launch_linear(X, Wg, Bg, T, H, E, dtype, scores, s);
     if (rc != OPMX_OK) return rc;
-    return launch_moe_select(X, scores, T, H, E, k, dtype, Xp, w, inv, off, ids, ws, s);
+    return launch_moe_select(X, scores, T, H, E, k, dtype, Xp, w, inv, off, ids, ws, s, row_token);
 }
 
 size_t moe_select_workspace_bytes(int64_t T, int E, int k)
@@ -553,12 +561,13 @@ size_t moe_select_workspace_bytes(int64_t T, int E, int k)
 }
 
 int launch_moe_select(const void *X, const void *scores, int64_t T, int64_t H, int E, int k, int dtype,
-                      void *Xp, void *w, int64_t *inv, int64_t *off, int32_t *ids, void *ws, hipStream_t s)
+                      void *Xp, void *w, int64_t *inv, int64_t *off, int32_t *ids, void *ws, hipStream_t s,
+                      int32_t *row_token)
 {
     switch (dtype) {
-        case OPMX_DTYPE_F32: return select_impl<float>(X, scores, T, H, E, k, Xp, w, inv, off, ids, ws, s);
-        case OPMX_DTYPE_F16: return select_impl<f16>(X, scores, T, H, E, k, Xp, w, inv, off, ids, ws, s);
-        case OPMX_DTYPE_BF16: return select_impl<bf16>(X, scores, T, H, E, k, Xp, w, inv, off, ids, ws, s);
+        case OPMX_DTYPE_F32: return select_impl<float>(X, scores, T, H, E, k, Xp, w, inv, off, ids, ws, s, row_token);
+        case OPMX_DTYPE_F16: return select_impl<f16>(X, scores, T, H, E, k, Xp, w, inv, off, ids, ws, s, row_token);
+        case OPMX_DTYPE_BF16: return select_impl<bf16>(X, scores, T, H, E, k, Xp, w, inv, off, ids, ws, s, row_token);
     }
     return OPMX_ERR_UNSUPPORTED;
 }
@@ -602,7 +611,7 @@ int launch_moe_select_static(const void *X, const void *scores, int64_t T, int64
     void *ws = nullptr;
     const int rc = scratch_for_current_device(&ws);
     if (rc != OPMX_OK) return rc;
-    return launch_moe_select(X, scores, T, H, E, k, dtype, Xp, w, inv, off, ids, ws, s);
+    return launch_moe_select(X, scores, T, H, E, k, dtype, Xp, w, inv, off, ids, ws, s, nullptr);
 }
 
 }  // namespace opmx

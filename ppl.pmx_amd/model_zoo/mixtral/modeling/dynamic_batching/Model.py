@@ -33,11 +33,17 @@ class MoeFeedForward(nn.Module):
     the operator-by-operator route.  ``fuse_router_select=True`` does the same for the router
     gate and MoeSelect (one launch up to 8 tokens; the routing is exact on the logits that
     launch computes, which can differ from the separate gate's in the last bit).
+    ``fuse_x_gather=True`` folds the token gather of MoeSelect (``MoeSelect.py:45-47``) into the
+    operand load of the gate/up GEMM: MoeSelect then returns an index instead of
+    ``X_expand_permute`` and the ``[T*k, H]`` copy is never written; same bits as the separate
+    operators.
     """
 
     def __init__(self, args, layer_id: int, fused_ffn_glu: bool, linear_bias_term: bool, proc_group,
-                 dtype=None, device=None, fuse_swiglu_epilogue: bool = False, fuse_router_select: bool = False):
+                 dtype=None, device=None, fuse_swiglu_epilogue: bool = False, fuse_router_select: bool = False,
+                 fuse_x_gather: bool = False):
         super().__init__()
+        self.fuse_x_gather = fuse_x_gather
         self.layer_id = layer_id
         self.fused_ffn_glu = fused_ffn_glu
         self.fuse_swiglu_epilogue = fuse_swiglu_epilogue and fused_ffn_glu
@@ -63,8 +69,27 @@ class MoeFeedForward(nn.Module):
         return SimpleNamespace(hidden_dim=hidden_dim, intermediate_dim=intermediate_dim,
                                num_experts=num_experts, num_experts_per_token=num_experts_per_token)
 
+    def _forward_indexed(self, x):
+        """The block with MoeSelect as an index (``fuse_x_gather``): same operator order as ``forward``."""
+        k, E = self.num_experts_per_token, self.num_experts
+        if self.fuse_router_select:
+            expert_weights, invert_permutation, expert_offset, row_token, _ = OPMX.moe_route_select_index(
+                x, self.gate.weight, self.gate.bias, E, k)
+        else:
+            expert_weights, invert_permutation, expert_offset, row_token = OPMX.moe_select_index(self.gate(x), E, k)
+        col = lambda m, swiglu=False: OPMX.moe_column_parallel_linear_indexed(
+            x, row_token, expert_offset, m.weight, m.bias, E, m.in_features, m.out_features, swiglu=swiglu)
+        if self.fused_ffn_glu:
+            x13 = col(self.wu, True) if self.fuse_swiglu_epilogue else OPMX.swiglu(col(self.wu))
+        else:
+            x13 = OPMX.silu(col(self.w1), col(self.w3))
+        x_out = self.w2(x13, expert_offset)
+        return OPMX.moe_reduce(x_out, expert_weights, invert_permutation, k)
+
     def forward(self, x):
         k = self.num_experts_per_token
+        if self.fuse_x_gather and not torch.onnx.is_in_onnx_export():
+            return self._forward_indexed(x)
         if self.fuse_router_select and not torch.onnx.is_in_onnx_export():
             x_experts, expert_weights, invert_permutation, expert_offset, _ = OPMX.moe_route_select(
                 x, self.gate.weight, self.gate.bias, self.num_experts, k)
@@ -176,7 +201,8 @@ class GraphedMoeFeedForward(nn.Module):
 
 
 def load_opmx_moe_block(path, layer_id: int, num_experts_per_token: int, fused_ffn_glu: bool = True,
-                        dtype=None, device=None, fuse_swiglu_epilogue: bool = False, fuse_router_select: bool = False):
+                        dtype=None, device=None, fuse_swiglu_epilogue: bool = False, fuse_router_select: bool = False,
+                        fuse_x_gather: bool = False):
     """Builds the MoE block of layer ``layer_id`` from an OPMX Mixtral ``.pth`` checkpoint.
 
     The file is opened with ``weights_only=True`` and memory-mapped, so only this layer's tensors are
@@ -191,6 +217,7 @@ def load_opmx_moe_block(path, layer_id: int, num_experts_per_token: int, fused_f
     bias = (prefix + "w2.bias") in sd
     block = MoeFeedForward(MoeFeedForward.params(H, w2.shape[2], E, num_experts_per_token), layer_id, fused_ffn_glu,
                            bias, None, dtype=gate.dtype if dtype is None else dtype, device=device,
-                           fuse_swiglu_epilogue=fuse_swiglu_epilogue, fuse_router_select=fuse_router_select)
+                           fuse_swiglu_epilogue=fuse_swiglu_epilogue, fuse_router_select=fuse_router_select,
+                           fuse_x_gather=fuse_x_gather)
     block.load_state_dict(sd)
     return block

@@ -49,3 +49,15 @@ def moe_column_parallel_linear_swiglu(X, expert_offset, W, B, num_experts: int, 
     of ``Model.py:198`` and ``Model.py:200``); eager only."""
     assert X.shape[-1] == in_features, "X.shape is {}, in_features is {}".format(X.shape, in_features)
     return grouped_linear("column", X, expert_offset, W, B, num_experts, epilogue=_lib.EPILOGUE_SWIGLU)
+
+
+def moe_column_parallel_linear_indexed(X, row_token, expert_offset, W, B, num_experts: int, in_features: int,
+                                       out_features: int, swiglu: bool = False) -> torch.Tensor:
+    """``moe_column_parallel_linear`` (or its SwiGLU form) on the rows ``X[row_token]``: ``X`` ``[*, K]``
+    holds the tokens, ``row_token`` is the int32 index ``moe_select_index`` returns in place of
+    ``X_expand_permute``.  Bit for bit the result of the operator on ``X_expand_permute``
+    (``MoeSelect.py:45-47`` followed by ``MoeColumnParallelLinear.py:58-67``), ``[*, k, N]``, without the
+    ``[T*k, K]`` copy ever being written or read.  No counterpart operator in the reference; eager only."""
+    assert X.shape[-1] == in_features, "X.shape is {}, in_features is {}".format(X.shape, in_features)
+    return grouped_linear("column", X, expert_offset, W, B, num_experts,
+                          epilogue=_lib.EPILOGUE_SWIGLU if swiglu else _lib.EPILOGUE_NONE, row_index=row_token)

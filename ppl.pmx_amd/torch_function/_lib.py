@@ -36,7 +36,12 @@ _SIGNATURES = {
     "opmx_moe_select_static": (_int, [_vp, _vp, _i64, _i64, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp]),
     "opmx_moe_route_select": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                      _sz, _vp]),
+    "opmx_moe_select_index": (_int, [_vp, _i64, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "opmx_moe_route_select_index": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp,
+                                           _vp, _sz, _vp]),
     "opmx_moe_grouped_gemm_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _int]),
+    "opmx_moe_column_parallel_linear_indexed": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _int,
+                                                       _i64, _vp, _vp, _sz, _vp]),
     "opmx_moe_column_parallel_linear": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _int, _i64,
                                                _vp, _vp, _sz, _vp]),
     "opmx_moe_row_parallel_linear": (_int, [_vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _i64,

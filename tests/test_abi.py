@@ -73,6 +73,20 @@ def test_argument_validation_needs_no_device(lib):
     assert rs(one, one, None, 4, 8, 8, 2, 1, one, one, one, one, one, None, None, 0, None) == -3        # workspace
     assert rs(one, None, None, 4, 8, 8, 2, 1, one, one, one, one, one, None, one, 1 << 20, None) == -1  # gate weight
     assert rs(one, one, None, 4, 8, 8, 2, 1, None, one, one, one, one, None, one, 1 << 20, None) == -1  # scores
+    # MoeSelect as an index, and the GEMM that reads its rows through it
+    si = lambda *a: lib.opmx_moe_select_index(*a)
+    assert si(one, 4, 8, 9, 1, one, one, one, one, None, one, 1 << 20, None) == -1      # k > E
+    assert si(one, 4, 300, 2, 1, one, one, one, one, None, one, 1 << 20, None) == -2    # E
+    assert si(one, 4, 8, 2, 1, one, one, one, None, None, one, 1 << 20, None) == -1     # no row_token
+    assert si(one, 4, 8, 2, 1, one, one, one, one, None, None, 0, None) == -3           # workspace
+    rsi = lambda *a: lib.opmx_moe_route_select_index(*a)
+    assert rsi(one, None, None, 4, 8, 8, 2, 1, one, one, one, one, one, None, one, 1 << 20, None) == -1   # gate weight
+    assert rsi(one, one, None, 4, 8, 8, 2, 1, one, one, one, one, None, None, one, 1 << 20, None) == -1   # no row_token
+    gi = lambda *a: lib.opmx_moe_column_parallel_linear_indexed(*a)
+    assert gi(one, 4, None, one, one, None, 8, 8, 64, 32, 1, 0, 0, one, None, 0, None) == -1    # no index
+    assert gi(one, 0, one, one, one, None, 8, 8, 64, 32, 1, 0, 0, one, None, 0, None) == -1     # X without rows
+    assert gi(one, 4, one, one, one, None, 8, 8, 64, 33, 1, 1, 0, one, None, 0, None) == -1     # SwiGLU needs an even N
+    assert gi(None, 0, None, None, None, None, 8, 0, 64, 32, 1, 0, 0, None, None, 0, None) == 0  # empty
     assert lib.opmx_moe_column_parallel_linear(one, one, one, None, 8, 4, 64, 33, 1, 1, 0, one, None, 0, None) == -1
     assert lib.opmx_moe_column_parallel_linear(one, None, one, None, 8, 4, 64, 32, 1, 0, 0, one, None, 0, None) == -1
     assert lib.opmx_moe_row_parallel_linear(one, one, one, None, 999, 4, 64, 32, 1, 0, one, None, 0, None) == -2
