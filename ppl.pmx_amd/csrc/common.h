@@ -119,6 +119,8 @@ int launch_linear(const void *X, const void *W, const void *B, int64_t T, int64_
                   int dtype, void *Y, hipStream_t s);
 // Xp == nullptr: routing only (no row copy); row_token (may be nullptr) receives, for every row of the
 // permuted order, the token whose copy it is.
+int launch_linear_route(const void *X, const void *W, const void *B, int64_t T, int64_t K, int E, int k, int dtype,
+                        void *scores, void *weights, int32_t *ids, hipStream_t s);
 int launch_moe_select(const void *X, const void *scores, int64_t T, int64_t H, int E, int k, int dtype,
                       void *Xp, void *w, int64_t *inv, int64_t *off, int32_t *ids, void *ws,
                       hipStream_t s, int32_t *row_token = nullptr);

@@ -3,6 +3,7 @@
 // tokens' rows once with 16-byte loads and keeps W in cache.
 // Semantics: torch_function/Linear.py:32 of OpenPPL/ppl.pmx.
 #include "moe_gemm.h"
+#include "moe_route.h"
 
 namespace opmx {
 namespace {
@@ -81,13 +82,19 @@ __global__ __launch_bounds__(256) void linear_kernel(const T *__restrict__ X, co
 // and feed the MFMA 16x16x32 units straight from global memory: X is read once, 64-byte pieces
 // of 16 rows per load with four steps in flight, W comes from cache.  The partial sums meet in
 // LDS and are added in wave order.  NE = 16-output tiles per token tile.
-template <typename T, int NE, int NW>
+// ROUTE: the block holds all N <= 64 logits of its 16 tokens (one block over the outputs), rounds
+// them, and goes on to route those tokens on the rounded values -- top-k, ties to the lower expert
+// id, softmax over the picks (MoeSelect.py:40-41) -- writing expert ids and weights next to the
+// logits: MoeSelect then starts from the picks and the logits are never read back.
+template <typename T, int NE, int NW, bool ROUTE>
 __global__ __launch_bounds__(NW * 64) void linear_skinny_mfma_kernel(const T *__restrict__ X, const T *__restrict__ W,
                                                                       const T *__restrict__ B, int64_t Ttok, int64_t K,
-                                                                      int64_t N, T *__restrict__ Y)
+                                                                      int64_t N, T *__restrict__ Y, int k,
+                                                                      T *__restrict__ weights, int32_t *__restrict__ ids)
 {
     using frag = typename Mfma<T>::frag;
     __shared__ __attribute__((aligned(16))) float part[NW * NE * 64 * 4];
+    __shared__ T s_scores[ROUTE ? 16 * NE * 16 : 1];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int fr = lane & 15, fg = lane >> 4;
     const int64_t t0 = static_cast<int64_t>(blockIdx.x) * 16;
@@ -136,7 +143,26 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_mfma_kernel(const T *__
 #pragma unroll
         for (int w = 0; w < NW; ++w) v += part[w * NE * 64 * 4 + idx];
         if (B) v += to_f32(B[n0 + n]);
-        Y[(t0 + t) * N + n0 + n] = from_f32<T>(v);
+        const T r = from_f32<T>(v);
+        Y[(t0 + t) * N + n0 + n] = r;
+        if (ROUTE) s_scores[t * static_cast<int>(N) + n] = r;
+    }
+    if (ROUTE) {
+        __syncthreads();
+        const int E = static_cast<int>(N);
+        int G = 8;
+        while (G < E) G <<= 1;                  // E <= 64: one key per lane
+        const int lig = threadIdx.x % G, grp = threadIdx.x / G, ngrp = NW * 64 / G;
+        for (int tl = grp; tl < 16; tl += ngrp) {            // whole lane groups iterate together
+            if (t0 + tl >= Ttok) break;
+            int id;
+            float w;
+            route_token(s_scores + tl * E, E, k, G, 1, lig, id, w);
+            if (lig < k) {
+                ids[(t0 + tl) * k + lig] = id;
+                weights[(t0 + tl) * k + lig] = from_f32<T>(w);
+            }
+        }
     }
 }
 
@@ -148,10 +174,27 @@ int linear_skinny_mfma(const void *X, const void *W, const void *B, int64_t Ttok
     const unsigned grid = static_cast<unsigned>(ceil_div(Ttok, 16));
     const T *x = static_cast<const T *>(X), *w = static_cast<const T *>(W), *b = static_cast<const T *>(B);
     T *y = static_cast<T *>(Y);
-    if (N <= 16) linear_skinny_mfma_kernel<T, 1, NW><<<grid, NW * 64, 0, s>>>(x, w, b, Ttok, K, N, y);
-    else if (N <= 32) linear_skinny_mfma_kernel<T, 2, NW><<<grid, NW * 64, 0, s>>>(x, w, b, Ttok, K, N, y);
+    if (N <= 16) linear_skinny_mfma_kernel<T, 1, NW, false><<<grid, NW * 64, 0, s>>>(x, w, b, Ttok, K, N, y, 0, nullptr, nullptr);
+    else if (N <= 32) linear_skinny_mfma_kernel<T, 2, NW, false><<<grid, NW * 64, 0, s>>>(x, w, b, Ttok, K, N, y, 0, nullptr, nullptr);
     else   // 64 outputs per block; more outputs: more blocks over the same tokens (X read once per 64 outputs)
-        linear_skinny_mfma_kernel<T, 4, NW><<<dim3(grid, static_cast<unsigned>(ceil_div(N, 64))), NW * 64, 0, s>>>(x, w, b, Ttok, K, N, y);
+        linear_skinny_mfma_kernel<T, 4, NW, false><<<dim3(grid, static_cast<unsigned>(ceil_div(N, 64))), NW * 64, 0, s>>>(
+            x, w, b, Ttok, K, N, y, 0, nullptr, nullptr);
+    OPMX_LAUNCH_CHECK();
+    return OPMX_OK;
+}
+
+// The same kernel with the routing of its tokens in the epilogue (N = number of experts <= 64).
+template <typename T>
+int linear_skinny_route(const void *X, const void *W, const void *B, int64_t Ttok, int64_t K, int64_t N, int k, void *Y,
+                        void *weights, int32_t *ids, hipStream_t s)
+{
+    constexpr int NW = 8;
+    const unsigned grid = static_cast<unsigned>(ceil_div(Ttok, 16));
+    const T *x = static_cast<const T *>(X), *w = static_cast<const T *>(W), *b = static_cast<const T *>(B);
+    T *y = static_cast<T *>(Y), *wt = static_cast<T *>(weights);
+    if (N <= 16) linear_skinny_mfma_kernel<T, 1, NW, true><<<grid, NW * 64, 0, s>>>(x, w, b, Ttok, K, N, y, k, wt, ids);
+    else if (N <= 32) linear_skinny_mfma_kernel<T, 2, NW, true><<<grid, NW * 64, 0, s>>>(x, w, b, Ttok, K, N, y, k, wt, ids);
+    else linear_skinny_mfma_kernel<T, 4, NW, true><<<grid, NW * 64, 0, s>>>(x, w, b, Ttok, K, N, y, k, wt, ids);
     OPMX_LAUNCH_CHECK();
     return OPMX_OK;
 }
@@ -184,6 +227,28 @@ int linear_impl(const void *X_, const void *W_, const void *B_, int64_t Ttok, in
 
 }  // namespace
 
+// Whether the router logits of T tokens over N experts go through linear_skinny_mfma_kernel
+// (measured crossovers against the other two kernels, see launch_linear).
+static bool skinny_mfma_pays(int64_t T, int64_t K, int64_t N, int dtype, const void *X, const void *W)
+{
+    return (dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16) && N <= 256 && K >= 32 && K % 32 == 0 && aligned16(X) &&
+           aligned16(W) &&
+           (N <= 8 ? T >= 4096 : N <= 64 ? (T >= 512 && (N <= 16 || T < 8192)) : (T * N >= 32768 && T * N <= 262144));
+}
+
+// Router logits and, in the same launch, the routing of every token on them: scores [T,E] as
+// launch_linear writes them, expert ids [T,k] and weights [T,k] as MoeSelect's top-k kernel writes
+// them.  Only where the skinny MFMA kernel is the router kernel anyway and one block holds a
+// token's E <= 64 logits; OPMX_ERR_UNSUPPORTED otherwise (nothing enqueued: the caller runs the
+// two operators one after the other).
+int launch_linear_route(const void *X, const void *W, const void *B, int64_t T, int64_t K, int E, int k, int dtype,
+                        void *scores, void *weights, int32_t *ids, hipStream_t s)
+{
+    if (E > 64 || k > E || !skinny_mfma_pays(T, K, E, dtype, X, W)) return OPMX_ERR_UNSUPPORTED;
+    return dtype == OPMX_DTYPE_F16 ? linear_skinny_route<f16>(X, W, B, T, K, E, k, scores, weights, ids, s)
+                                   : linear_skinny_route<bf16>(X, W, B, T, K, E, k, scores, weights, ids, s);
+}
+
 int launch_linear(const void *X, const void *W, const void *B, int64_t T, int64_t K, int64_t N, int dtype,
                   void *Y, hipStream_t s)
 {
@@ -196,9 +261,7 @@ int launch_linear(const void *X, const void *W, const void *B, int64_t T, int64_
     // in four blocks of 64 over the same tokens: 37 us against 64 up to T = 1024, 71 against 64 at 2048;
     // its K chain costs about H / 195 us whatever T is, which one block per token undercuts up to
     // T * N of about 32768: 256 outputs, T = 128: 31 us per-token blocks, 36 us this kernel; T = 256: 61 / 37).
-    if ((dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16) && N <= 256 && K >= 32 && K % 32 == 0 && aligned16(X) &&
-        aligned16(W) &&
-        (N <= 8 ? T >= 4096 : N <= 64 ? (T >= 512 && (N <= 16 || T < 8192)) : (T * N >= 32768 && T * N <= 262144)))
+    if (skinny_mfma_pays(T, K, N, dtype, X, W))
         return dtype == OPMX_DTYPE_F16 ? linear_skinny_mfma<f16>(X, W, B, T, K, N, Y, s)
                                        : linear_skinny_mfma<bf16>(X, W, B, T, K, N, Y, s);
     if ((dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16) && T >= 512 && N > 8 && K % 64 == 0 &&

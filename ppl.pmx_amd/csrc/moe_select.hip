@@ -9,130 +9,13 @@
 #include <mutex>
 
 #include "moe_gemm.h"
+#include "moe_route.h"
 
 namespace opmx {
 namespace {
 
 constexpr int kChunk = 256;          // tokens per routing block
 constexpr int kWords = kChunk / 32;  // bit-matrix words per expert
-constexpr int kMaxVpl = OPMX_MOE_MAX_EXPERTS / kWave;
-
-// Monotone map float -> uint32 (larger float => larger key).  NaN is the
-// largest key (torch.topk / torch.sort rank NaN first); -0.0 == +0.0.
-__device__ __forceinline__ uint32_t order_key(float f)
-{
-    if (f != f) return 0xFFFFFFFFu;
-    if (f == 0.0f) f = 0.0f;
-    uint32_t u = __float_as_uint(f);
-    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-}
-__device__ __forceinline__ float key_value(uint32_t key)
-{
-    if (key == 0xFFFFFFFFu) return __uint_as_float(0x7FC00000u);
-    uint32_t u = (key & 0x80000000u) ? (key & 0x7FFFFFFFu) : ~key;
-    return __uint_as_float(u);
-}
-
-__device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int mask)
-{
-    uint32_t lo = __shfl_xor(static_cast<uint32_t>(v), mask, kWave);
-    uint32_t hi = __shfl_xor(static_cast<uint32_t>(v >> 32), mask, kWave);
-    return (static_cast<uint64_t>(hi) << 32) | lo;
-}
-
-// One group of G lanes (G a power of two, 8..64) routes one token.  Lane j < k
-// of the group ends up with the j-th pick and its softmax weight.
-template <typename T>
-__device__ __forceinline__ void route_token(const T *srow, int E, int k, int G, int vpl, int lig,
-                                            int &my_id, float &my_w)
-{
-    uint64_t keys[kMaxVpl];
-#pragma unroll
-    for (int v = 0; v < kMaxVpl; ++v) {
-        int e = lig + v * G;
-        keys[v] = (v < vpl && e < E)
-                      ? (static_cast<uint64_t>(order_key(to_f32(srow[e]))) << 32) | (0xFFFFFFFFu - e)
-                      : 0ull;
-    }
-    my_id = -1;
-    float my_v = 0.0f;
-    // With several keys per lane (E > 64) the ranking below costs E broadcasts of up to four
-    // compares each; the k rounds of the other branch are cheaper there (E = 256, k = 8: MoeSelect at
-    // T = 512 51 -> 38 us, at T = 8192 291 -> 247 us), so only one key per lane is ranked.
-    if (G == kWave && vpl == 1) {
-        // A whole wave routes the token.  Keys are distinct (the id is part of the key),
-        // so "how many keys beat mine" is the key's position in the descending order:
-        // E scalar broadcasts and compares, no k-round dependency chain.  The key of
-        // rank j then moves to lane j through LDS-free cross-lane reads.
-        int rank[kMaxVpl];
-#pragma unroll
-        for (int v = 0; v < kMaxVpl; ++v) rank[v] = 0;
-        if (vpl == 1) {                      // E <= 64: one key per lane
-            for (int sl = 0; sl < E; ++sl) {
-                const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[0]), sl);
-                const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[0] >> 32), sl);
-                rank[0] += ((static_cast<uint64_t>(hi) << 32) | lo) > keys[0] ? 1 : 0;
-            }
-        } else {
-#pragma unroll
-            for (int sv = 0; sv < kMaxVpl; ++sv) {
-                if (sv < vpl) {
-                    for (int sl = 0; sl < kWave; ++sl) {
-                        if (sl + sv * kWave >= E) break;
-                        const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[sv]), sl);
-                        const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[sv] >> 32), sl);
-                        const uint64_t other = (static_cast<uint64_t>(hi) << 32) | lo;
-#pragma unroll
-                        for (int v = 0; v < kMaxVpl; ++v) rank[v] += other > keys[v] ? 1 : 0;
-                    }
-                }
-            }
-        }
-        // lane j < k fetches the key whose rank is j: every lane publishes (rank -> key) by ballot
-#pragma unroll
-        for (int v = 0; v < kMaxVpl; ++v) {
-            if (v < vpl) {
-                for (int j = 0; j < k; ++j) {
-                    const uint64_t hit = __ballot(rank[v] == j && keys[v] != 0ull);
-                    if (hit) {
-                        const int src = __ffsll(static_cast<long long>(hit)) - 1;
-                        const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[v]), src);
-                        const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[v] >> 32), src);
-                        if (lig == j) {
-                            my_id = static_cast<int>(0xFFFFFFFFu - lo);
-                            my_v = key_value(hi);
-                        }
-                    }
-                }
-            }
-        }
-    } else {
-        for (int j = 0; j < k; ++j) {
-            uint64_t best = keys[0];
-#pragma unroll
-            for (int v = 1; v < kMaxVpl; ++v) best = keys[v] > best ? keys[v] : best;
-            for (int m = G >> 1; m >= 1; m >>= 1) {
-                uint64_t o = shfl_xor_u64(best, m);
-                best = o > best ? o : best;
-            }
-            int wid = static_cast<int>(0xFFFFFFFFu - static_cast<uint32_t>(best));
-#pragma unroll
-            for (int v = 0; v < kMaxVpl; ++v)
-                if (lig + v * G == wid) keys[v] = 0ull;
-            if (lig == j) {
-                my_id = wid;
-                my_v = key_value(static_cast<uint32_t>(best >> 32));
-            }
-        }
-    }
-    // softmax over the k picked values (MoeSelect.py:41); pick 0 is the maximum
-    float vmax = __shfl(my_v, (lane_id() / G) * G, kWave);
-    float ev = (lig < k) ? expf(my_v - vmax) : 0.0f;
-    float sum = ev;
-    for (int m = G >> 1; m >= 1; m >>= 1) sum += __shfl_xor(sum, m, kWave);
-    my_w = ev / sum;
-}
-
 __device__ __forceinline__ void zero_bits(uint32_t *bits, int E)
 {
     for (int i = threadIdx.x; i < E * kWords; i += blockDim.x) bits[i] = 0u;
@@ -452,6 +335,15 @@ __global__ __launch_bounds__(1024) void select_small_kernel(const T *__restrict_
     expand_row(X, Xp, static_cast<int64_t>(me), H, k, my_inv, vec);
 }
 
+// The buffer select_impl keeps the picked ids in: the caller's, or a part of the workspace.
+inline int32_t *picks_buffer(int64_t Ttok, int E, int32_t *ids, void *ws)
+{
+    const int nchunks = static_cast<int>(ceil_div(Ttok, kChunk));
+    return ids ? ids : reinterpret_cast<int32_t *>(static_cast<char *>(ws) + ceil_div(sizeof(int32_t) * nchunks * E, 256) * 256);
+}
+
+// scores_ == nullptr (more than kChunk tokens only): the picks are made -- expert ids in
+// picks_buffer(), weights in w_ -- and the top-k kernel is skipped.
 template <typename T>
 int select_impl(const void *X_, const void *scores_, int64_t Ttok, int64_t H, int E, int k, void *Xp_, void *w_,
                 int64_t *inv, int64_t *off, int32_t *ids, void *ws, hipStream_t s, int32_t *row_token)
@@ -486,7 +378,7 @@ int select_impl(const void *X_, const void *scores_, int64_t Ttok, int64_t H, in
     const int nchunks = static_cast<int>(ceil_div(Ttok, kChunk));
     char *wsb = static_cast<char *>(ws);
     int32_t *hist = reinterpret_cast<int32_t *>(wsb);
-    int32_t *idbuf = ids ? ids : reinterpret_cast<int32_t *>(wsb + ceil_div(sizeof(int32_t) * nchunks * E, 256) * 256);
+    int32_t *idbuf = picks_buffer(Ttok, E, ids, ws);
     if (Ttok <= kChunk) {
         select_topk_kernel<T><<<static_cast<unsigned>(ceil_div(Ttok, kChunk / G)), kChunk, 0, s>>>(scores, Ttok, E, k, G,
                                                                                                    vpl, w, idbuf);
@@ -496,9 +388,11 @@ int select_impl(const void *X_, const void *scores_, int64_t Ttok, int64_t H, in
         OPMX_LAUNCH_CHECK();
         return OPMX_OK;
     }
-    select_topk_kernel<T><<<static_cast<unsigned>(ceil_div(Ttok, kChunk / G)), kChunk, 0, s>>>(scores, Ttok, E, k, G,
-                                                                                               vpl, w, idbuf);
-    OPMX_LAUNCH_CHECK();
+    if (scores != nullptr) {
+        select_topk_kernel<T><<<static_cast<unsigned>(ceil_div(Ttok, kChunk / G)), kChunk, 0, s>>>(scores, Ttok, E, k, G,
+                                                                                                   vpl, w, idbuf);
+        OPMX_LAUNCH_CHECK();
+    }
     select_hist_kernel<<<nchunks, kChunk, 0, s>>>(idbuf, Ttok, E, k, hist);
     OPMX_LAUNCH_CHECK();
     select_scan_kernel<<<1, E > 16 ? 1024 : 256, 0, s>>>(hist, nchunks, E, R, off);
@@ -547,6 +441,11 @@ int launch_moe_route_select(const void *X, const void *Wg, const void *Bg, int64
             return route_select_fused<f16>(X, Wg, Bg, T, H, E, k, scores, Xp, w, inv, off, ids, s, row_token);
         return route_select_fused<bf16>(X, Wg, Bg, T, H, E, k, scores, Xp, w, inv, off, ids, s, row_token);
     }
+    // Many tokens, few experts: the router kernel that holds a token's logits in one block routes
+    // it as well, and MoeSelect starts from the picks (one launch and the read-back of the logits less).
+    if (T > kChunk &&
+        launch_linear_route(X, Wg, Bg, T, H, E, k, dtype, scores, w, picks_buffer(T, E, ids, ws), s) == OPMX_OK)
+        return launch_moe_select(X, nullptr, T, H, E, k, dtype, Xp, w, inv, off, ids, ws, s, row_token);
     const int rc = launch_linear(X, Wg, Bg, T, H, E, dtype, scores, s);
     if (rc != OPMX_OK) return rc;
     return launch_moe_select(X, scores, T, H, E, k, dtype, Xp, w, inv, off, ids, ws, s, row_token);

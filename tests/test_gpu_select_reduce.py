@@ -221,7 +221,13 @@ ROUTE_SELECT_CASES = [
     (8, 2048, 64, 8, torch.bfloat16, False),    # too many experts
     (8, 100, 8, 2, torch.float16, True),        # H not a multiple of 32
     (8, 64, 8, 2, torch.float32, True),         # fp32
-    (600, 512, 16, 2, torch.float16, False),    # long prompt: tiled router GEMM + general select
+    (600, 512, 16, 2, torch.float16, False),    # long prompt, 16 experts: the router kernel routes in its epilogue
+    (4096, 512, 8, 2, torch.float16, True),     # 8 experts from 4096 tokens on: router kernel with routing epilogue
+    (4100, 256, 8, 2, torch.bfloat16, False),   # ... a last block with 4 tokens
+    (1000, 2048, 64, 8, torch.bfloat16, False), # 64 experts, top-8: one key per lane of a whole wave
+    (700, 256, 33, 5, torch.float16, True),     # 33 experts: three 16-output tiles, the last one ragged
+    (520, 256, 64, 32, torch.float16, False),   # limits of the routing epilogue: 64 experts, 32 picks
+    (300, 512, 16, 2, torch.float16, False),    # below 512 tokens: the two operators one after the other
 ]
 
 
