@@ -84,7 +84,6 @@ const char *opmx_status_string(int status);
  *   "OPMX_MOE_GEMM_GNX"            tile order: 8 expert-major, 16 row partition, 4, 0 row-major
  *   "OPMX_MOE_GEMM_STREAMK"        0 never split the tail tiles over K, 2 whenever possible
  *   "OPMX_MOE_GEMM_PERSIST"        0 never the persistent form, 1 whenever its conditions hold
- *   "OPMX_MOE_GEMM_RAGGED"         0 never the short forms of the k loop for ragged tiles, 1 always
  * Returns OPMX_ERR_BAD_ARGUMENT for an unknown name. */
 int opmx_moe_set_option(const char *name, int value);
 

@@ -11,9 +11,8 @@ checked on its output instead:
 2. no buffer load sits in a loop over lanes (a descriptor the compiler cannot prove uniform), and
    nothing spills to scratch memory inside the k loop: both would add memory operations the
    hand-written `s_waitcnt vmcnt(N)` counts know nothing about;
-3. every k loop (the innermost loops with MFMAs, by the compiler's loop annotations) holds exactly
-   the MFMAs, LDS reads and loads of one k-tile in one of the four forms of the tile (8, 6, 4 or 2
-   sub-tiles per wave);
+3. the k loop (the loop with the most MFMAs, by the compiler's loop annotations) holds exactly
+   the MFMAs, LDS reads and loads of one k-tile;
 4. the persistent kernel issues the number of output stores per tile that its wait counts assume,
    and its tile loop has no scratch access and no wait that would drain the pipeline.
 
@@ -108,27 +107,14 @@ def check(path):
         khead = max((h for h in per_loop if h in innermost),
                     key=lambda h: sum(x.startswith("v_mfma") for x in per_loop[h]), default=None)
         kloop = per_loop.get(khead, [])
-        # The k loop exists in four forms, for tiles that need 8, 6, 4 or 2 of a wave's eight 16-row
-        # sub-tiles: MFMAs and X fragment reads of the other sub-tiles are left out, loads are not
-        # (inside the loop of the 2-sub-tile form two of the next k-tile's first X fragments are dead as well).
-        # 256 x 256 tiles (template arguments <T, 256, 256, ...>) or 128 x 256.
-        forms = ({(64, 24, 12), (48, 20, 12), (32, 16, 12), (16, 12, 12)} if "Li128ELi256E" in name
-                 else {(128, 32, 16), (96, 28, 16), (64, 24, 16), (32, 20, 16)})
-        seen_forms = set()
-        for h in sorted(innermost):
-            body_h = per_loop.get(h, [])
-            cnt = lambda p: sum(x.startswith(p) for x in body_h)
-            if cnt("v_mfma") == 0:
-                continue
-            form = (cnt("v_mfma"), cnt("ds_read_b128"), cnt("buffer_load_dwordx4"))
-            if form not in forms:
-                findings.append((name, "a k loop holds {} MFMAs, {} LDS reads, {} loads (expected one of {})".format(
-                    *form, sorted(forms, reverse=True))))
-            seen_forms.add(form)
-            if any(x.startswith("scratch_") for x in body_h):
-                findings.append((name, "scratch access inside a k loop"))
-        if max(forms) not in seen_forms:
-            findings.append((name, "no k loop of full tiles found"))
+        count = lambda p: sum(x.startswith(p) for x in kloop)
+        # 256 x 256 tiles (template arguments <T, 256, 256, ...>) or 128 x 256
+        expected = (64, 24, 12) if "Li128ELi256E" in name else (128, 32, 16)
+        if (count("v_mfma"), count("ds_read_b128"), count("buffer_load_dwordx4")) != expected:
+            findings.append((name, "k loop holds {} MFMAs, {} LDS reads, {} loads (expected {}, {}, {})".format(
+                count("v_mfma"), count("ds_read_b128"), count("buffer_load_dwordx4"), *expected)))
+        if any(x.startswith("scratch_") for x in kloop):
+            findings.append((name, "scratch access inside the k loop"))
         # 4. persistent kernel: the wait counts assume a fixed number of output stores per wave and
         #    tile (16 or 32), the same number of priming stores before the tile loop, and no other
         #    store in the loop
@@ -146,8 +132,7 @@ def check(path):
                 tile = [l for l, h in zip(text, where) if inside(h)]
                 rest = [l for l, h in zip(text, where) if not inside(h)]
                 st = lambda part: sum(x.startswith("buffer_store_dwordx4") for x in part)
-                # (the tile loop holds one copy of the epilogue per form of the k loop, or a single one)
-                if st(rest) not in (16, 32) or st(tile) not in (st(rest), 4 * st(rest)):
+                if st(rest) not in (16, 32) or st(tile) != st(rest):
                     findings.append((name, "{} priming stores, {} stores in the tile loop".format(st(rest), st(tile))))
                 # ... and that nothing in the tile loop drains the loads and stores kept in flight
                 # across tiles: no scratch traffic, no wait for all vector-memory operations

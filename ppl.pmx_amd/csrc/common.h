@@ -81,7 +81,6 @@ enum Option {
     kOptGnx,             // OPMX_MOE_GEMM_GNX: tile order 0 / 4 / 8 / 16
     kOptStreamK,         // OPMX_MOE_GEMM_STREAMK: 0 never split the tail tiles over K, 2 whenever possible
     kOptPersist,         // OPMX_MOE_GEMM_PERSIST: 0 never the persistent form, 1 whenever possible
-    kOptRagged,          // OPMX_MOE_GEMM_RAGGED: 0 never the short forms of the k loop for ragged tiles, 1 always
     kNumOptions
 };
 int option(Option o);

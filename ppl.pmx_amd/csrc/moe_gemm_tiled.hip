@@ -21,7 +21,6 @@
 // Semantics: torch_function/MoeColumnParallelLinear.py:61-67,
 // torch_function/MoeRowParallelLinear.py:47-53, torch_function/SwiGLU.py:15-16.
 #include <cstdlib>
-#include <type_traits>
 
 #include "moe_gemm.h"
 
@@ -304,16 +303,7 @@ inline int64_t linear_ids(int gnx, int ntiles_m, int ntiles_n)
 // Writes a wave's accumulators.  acc[j][i][v] is output row (X row) i*16 + lane%16 and output
 // column j*16 + (lane/16)*4 + v of the WTM x WTN wave tile: four consecutive columns per lane,
 // stored as one 8-byte word.  With SWIGLU sub-tiles j and j + TNS/2 hold gate and up columns.
-// ILV: how a wave's 16-row sub-tiles lie in the tile.  0: wave row wm owns the WTM consecutive rows
-// from wm * WTM on.  ILV > 0 (the number of wave rows): sub-tile i of wave row wm is the tile's
-// sub-tile i * ILV + wm -- the wave rows interleave, so that the rows a ragged tile does hold are
-// spread evenly over them (see tile_subtiles).
-template <int WTM, int ILV> __device__ __forceinline__ constexpr int wave_subtile_row(int wm, int i)
-{
-    return ILV > 0 ? (i * ILV + wm) * 16 : wm * WTM + i * 16;
-}
-
-template <typename T, int WTM, int WTN, bool SWIGLU, int ILV = 0>
+template <typename T, int WTM, int WTN, bool SWIGLU>
 __device__ __forceinline__ void tile_epilogue(float4_t (&acc)[WTN / 16][WTM / 16], const T *__restrict__ Bias,
                                               T *__restrict__ Y, const MTile &mt, int64_t N, int64_t ncols,
                                               int64_t n0, int wm, int wn, int lane)
@@ -324,7 +314,7 @@ __device__ __forceinline__ void tile_epilogue(float4_t (&acc)[WTN / 16][WTM / 16
     const bool vec_ok = (ncols % 4 == 0) && (reinterpret_cast<uintptr_t>(Y) % 8 == 0);
 #pragma unroll
     for (int i = 0; i < TMS; ++i) {
-        const int row = wave_subtile_row<WTM, ILV>(wm, i) + lrow;
+        const int row = wm * WTM + i * 16 + lrow;
         if (row >= mt.rows) continue;
         T *yrow = Y + (mt.row0 + row) * ncols;
 #pragma unroll
@@ -367,7 +357,7 @@ __device__ __forceinline__ void tile_epilogue(float4_t (&acc)[WTN / 16][WTM / 16
 // the lane's columns, and the swizzled LDS addresses (a staged row is at most 16 chunks and
 // sub-tiles start at multiples of 16 rows, so row % chunks == (lane % 16) % chunks for every
 // i and the row part of the address is an instruction offset).
-template <typename T, int WTM, int WTN, bool SWIGLU, bool BIAS, int ILV>
+template <typename T, int WTM, int WTN, bool SWIGLU, bool BIAS>
 __device__ __forceinline__ void tile_epilogue_lds_impl(float4_t (&acc)[WTN / 16][WTM / 16], const T *__restrict__ be,
                                                        T *__restrict__ Y, const MTile &mt, int64_t ncols, int64_t nw0,
                                                        int wm, int lane, char *wave_lds)
@@ -415,15 +405,12 @@ __device__ __forceinline__ void tile_epilogue_lds_impl(float4_t (&acc)[WTN / 16]
         }
     }
 
-    // read back whole rows: lane reads chunk c of staged row rr*RPI + lane/CH16.  Staged row s is
-    // row s % 16 of the wave's sub-tile s / 16 (an access never straddles sub-tiles: RPI divides 16).
-    static_assert(16 % RPI == 0, "an access covers rows of one sub-tile");
+    // read back whole rows: lane reads chunk c of row rr*RPI + lane/CH16
     const int c = lane % CH16, r0 = lane / CH16;
     const int64_t n = nw0 + c * 8;
     const bool col_ok = n < ncols;             // ncols % 8 == 0: a chunk is inside or outside as a whole
-    const int first = wave_subtile_row<WTM, ILV>(wm, 0) + r0;          // tile row of staged row r0
-    T *yp = Y + (mt.row0 + first) * ncols + n;
-    const int rows_left = static_cast<int>(mt.rows) - first;           // tile row first + d is stored iff d < rows_left
+    T *yp = Y + (mt.row0 + wm * WTM + r0) * ncols + n;
+    const int rows_left = static_cast<int>(mt.rows) - wm * WTM - r0;   // row rr*RPI is stored iff rr*RPI < rows_left
     constexpr int NR = WTM / RPI, BATCH = NR < 8 ? NR : 8;   // LDS reads in flight before their stores
 #pragma unroll
     for (int r8 = 0; r8 < NR; r8 += BATCH) {
@@ -435,24 +422,23 @@ __device__ __forceinline__ void tile_epilogue_lds_impl(float4_t (&acc)[WTN / 16]
         }
 #pragma unroll
         for (int u = 0; u < BATCH; ++u) {
-            const int s0 = (r8 + u) * RPI;                                      // staged row of lane group 0
-            const int d = wave_subtile_row<WTM, ILV>(0, s0 / 16) + s0 % 16;     // its distance from `first`, in tile rows
-            if (col_ok && d < rows_left) *reinterpret_cast<u32x4 *>(yp + static_cast<int64_t>(d) * ncols) = v[u];
+            if (col_ok && (r8 + u) * RPI < rows_left) *reinterpret_cast<u32x4 *>(yp) = v[u];
+            yp += static_cast<int64_t>(RPI) * ncols;
         }
     }
 }
 
-template <typename T, int WTM, int WTN, bool SWIGLU, int ILV = 0>
+template <typename T, int WTM, int WTN, bool SWIGLU>
 __device__ __forceinline__ void tile_epilogue_lds(float4_t (&acc)[WTN / 16][WTM / 16], const T *__restrict__ Bias,
                                                   T *__restrict__ Y, const MTile &mt, int64_t N, int64_t ncols,
                                                   int64_t n0, int wm, int wn, int lane, char *wave_lds)
 {
     const int64_t nw0 = (SWIGLU ? n0 + wn * (WTN / 2) : n0 + wn * WTN);   // first output column of this wave
     if (Bias)
-        tile_epilogue_lds_impl<T, WTM, WTN, SWIGLU, true, ILV>(acc, Bias + static_cast<int64_t>(mt.e) * N, Y, mt, ncols,
-                                                               nw0, wm, lane, wave_lds);
+        tile_epilogue_lds_impl<T, WTM, WTN, SWIGLU, true>(acc, Bias + static_cast<int64_t>(mt.e) * N, Y, mt, ncols, nw0,
+                                                          wm, lane, wave_lds);
     else
-        tile_epilogue_lds_impl<T, WTM, WTN, SWIGLU, false, ILV>(acc, nullptr, Y, mt, ncols, nw0, wm, lane, wave_lds);
+        tile_epilogue_lds_impl<T, WTM, WTN, SWIGLU, false>(acc, nullptr, Y, mt, ncols, nw0, wm, lane, wave_lds);
 }
 
 // Register-staged kernel: two LDS buffers, ONE register set staging global -> LDS, one barrier
@@ -838,23 +824,6 @@ __host__ __device__ inline int sk_split(int64_t ttot, int sk_wgs, int nk, int gn
     return (g - 1) * nk > cost * g ? g : 1;
 }
 
-// Ragged tiles.  An expert's last row tile holds fewer rows than the tile is high (on average half:
-// 7 % of all MFMA work at T = 8192 on the Mixtral shape, 24 % at T = 2048, 25 % with 64 experts at
-// T = 4096).  The wave rows of the direct-to-LDS kernels interleave (wave_subtile_row), so the rows
-// that are there are spread evenly over all waves, sub-tile by sub-tile from the top, and a tile
-// with few rows needs only the first `n` 16-row sub-tiles of EVERY wave.  The k loop exists in four
-// forms that issue the MFMAs (and read the X fragments) of the first 2, 4, 6 or 8 sub-tiles only --
-// compile-time variants chosen once per tile by a scalar branch, not a test per MFMA (which costs a
-// third of the speed of full tiles).  Loads, barriers and waits are the same in all four.
-// Returns n (even, 2 ... 8) for a tile of `rows` rows and WM wave rows.
-__device__ __forceinline__ int tile_subtiles(int rows, int WM)
-{
-    const int sub16 = (rows + 15) >> 4;                     // 16-row sub-tiles of the tile that hold rows
-    int n = (sub16 + WM - 1) / WM;                          // ... of wave row 0, which has the most
-    n = (n + 1) & ~1;
-    return __builtin_amdgcn_readfirstlane(n < 2 ? 2 : (n > 8 ? 8 : n));
-}
-
 // ---------------------------------------------------------------------------------------
 // Direct-to-LDS, 4 waves, fragments of a whole k-tile held in registers.  Each wave reads all
 // 32 fragments of k-tile kt (128 VGPRs) by the first third of the k-tile, so the LDS buffer is
@@ -898,7 +867,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
                                                                int64_t K, int64_t N, T *__restrict__ Y,
                                                                int ntiles_n, int gnx, int sk_wgs, int sk_cost,
                                                                float *__restrict__ sk_part, int *__restrict__ sk_count,
-                                                               const int32_t *__restrict__ rt, int64_t xrows, int forms)
+                                                               const int32_t *__restrict__ rt, int64_t xrows)
 {
     constexpr int NW = 4, WM = BM / 128, WN = NW / WM;                 // 256 x 256: 2 x 2 waves, 128 x 256: 1 x 4
     constexpr int WTM = BM / WM, WTN = BN / WN, TMS = WTM / 16, TNS = WTN / 16, HM = TMS / 2;
@@ -974,12 +943,10 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
 
     const int lrow = lane & 15, lk = lane >> 4;
     const int swz = (lrow >> 1) & 7;
-    constexpr int XSTEP = 16 * WM * ROWB;            // LDS bytes between a wave's consecutive X sub-tiles (interleaved wave rows)
-    const int x_off = (wm * 16 + lrow) * ROWB;
+    const int x_off = (wm * WTM + lrow) * ROWB;
     const int w_off = BM * ROWB + (wn * WTN + lrow) * ROWB;
     const int co0 = ((lk ^ swz) << 4), co1 = (((4 + lk) ^ swz) << 4);
     frag xf[2][2][HM], wf[2][TNS];      // [k32 step][X half][sub-tile], [k32 step][sub-tile]
-    const int nsub = forms ? tile_subtiles(mt.rows, WM) : 8;     // forms == 0: every tile takes the full form
 
     // wave load Q of k-tile KT into buffer BUF: Q < LA -> X rows, else W rows
 #define OPMX_ISSUE1(KT, BUF, Q)                                                                    \
@@ -991,78 +958,51 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
         else load_to_lds_16(rw, st_ + b_lds + ((Q)-LA) * 1024, b_src[(Q) < LA ? 0 : (Q)-LA], kb_); \
     } while (0)
 #define OPMX_XFRAG(BUF, S, H, I)                                                                   \
-    xf[S][H][I] = *reinterpret_cast<const frag *>(smem + (BUF)*STAGE + ((S) ? co1 : co0) + x_off + ((H)*HM + (I)) * XSTEP)
-    // the same when the tile's form (NS sub-tiles per wave, see tile_subtiles) multiplies that sub-tile
-#define OPMX_XFRAGN(NSB, BUF, S, H, I)                                                              \
-    do {                                                                                           \
-        if ((H)*HM + (I) < (NSB)) OPMX_XFRAG(BUF, S, H, I);                                         \
-    } while (0)
+    xf[S][H][I] = *reinterpret_cast<const frag *>(smem + (BUF)*STAGE + ((S) ? co1 : co0) + x_off + ((H)*HM + (I)) * 16 * ROWB)
 #define OPMX_WFRAG(BUF, S, J)                                                                      \
     wf[S][J] = *reinterpret_cast<const frag *>(smem + (BUF)*STAGE + ((S) ? co1 : co0) + w_off + (J)*16 * ROWB)
 #define OPMX_MF(S, H, m) Mfma<T>::m16_acc(wf[S][(m) % TNS], xf[S][H][(m) / TNS], acc[(m) % TNS][(H)*HM + (m) / TNS])
-    // MFMA m of X half H in the form with NSB sub-tiles per wave: only if its sub-tile is one of them
-#define OPMX_MFN(NSB, S, H, m)                                                                      \
-    do {                                                                                           \
-        if ((H)*HM + (m) / TNS < (NSB)) OPMX_MF(S, H, m);                                           \
-    } while (0)
     // the first k-tile of a tile overwrites the accumulators instead of adding to them
-#define OPMX_MF0(NSB, FIRST, H, m)                                                                  \
+#define OPMX_MF0(FIRST, H, m)                                                                      \
     do {                                                                                           \
-        if ((H)*HM + (m) / TNS < (NSB)) {                                                           \
-            if (FIRST) Mfma<T>::m16_first(wf[0][(m) % TNS], xf[0][H][(m) / TNS], acc[(m) % TNS][(H)*HM + (m) / TNS]); \
-            else OPMX_MF(0, H, m);                                                                 \
-        }                                                                                          \
+        if (FIRST) Mfma<T>::m16_first(wf[0][(m) % TNS], xf[0][H][(m) / TNS], acc[(m) % TNS][(H)*HM + (m) / TNS]); \
+        else OPMX_MF(0, H, m);                                                                     \
     } while (0)
     // One k-tile, held in buffer B.  LD2: load k-tile LDK (of this tile: two k-tiles ahead; or one
     // of the first two of the workgroup's next tile) into buffer B once it is free, then wait
     // until at most VM vector-memory operations are outstanding; without LD2 wait for all.
     // NEXT: read the first fragments of the following k-tile from the other buffer.
-    // NSB: the tile's form (tile_subtiles): MFMAs and X fragment reads of sub-tiles >= NSB are left
-    // out.  The first fragments of the FOLLOWING k-tile (group 3) are read whatever NSB is: it may
-    // belong to the workgroup's next tile, whose form can be another.
-#define OPMX_ITERX(NSB, LDK, B, LD2, NEXT, FIRST, VM)                                               \
+#define OPMX_ITERX(LDK, B, LD2, NEXT, FIRST, VM)                                                   \
     do {                                                                                           \
         _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
-            OPMX_MF0(NSB, FIRST, 0, m);                                                             \
+            OPMX_MF0(FIRST, 0, m);                                                                 \
             if (g0_reads(WIDE, m)) {                                                               \
                 const int r = g0_slot(WIDE, m);                                                    \
-                if (r < 4) OPMX_XFRAGN(NSB, B, 0, 1, r < 4 ? r : 0);                                \
-                else if (r < 8) OPMX_XFRAGN(NSB, B, 1, 0, (r >= 4 && r < 8) ? r - 4 : 0);           \
+                if (r < 4) OPMX_XFRAG(B, 0, 1, r < 4 ? r : 0);                                     \
+                else if (r < 8) OPMX_XFRAG(B, 1, 0, (r >= 4 && r < 8) ? r - 4 : 0);                \
                 else OPMX_WFRAG(B, 1, (r >= 8 && r < 8 + TNS) ? r - 8 : 0);                        \
             }                                                                                      \
         }                                                                                          \
         _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
-            OPMX_MF0(NSB, FIRST, 1, m);                                                             \
-            if (m < 4) OPMX_XFRAGN(NSB, B, 1, 1, m < 4 ? m : 0);                                    \
+            OPMX_MF0(FIRST, 1, m);                                                                 \
+            if (m < 4) OPMX_XFRAG(B, 1, 1, m < 4 ? m : 0);                                         \
             if (m == g1_barrier(WIDE)) barrier_no_fence();                                         \
             if ((LD2) && g1_load(WIDE, m) >= 0) OPMX_ISSUE1(LDK, B, g1_load(WIDE, m) >= 0 ? g1_load(WIDE, m) : 0); \
         }                                                                                          \
         _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
-            OPMX_MFN(NSB, 1, 0, m);                                                                 \
+            OPMX_MF(1, 0, m);                                                                      \
             if ((LD2) && g2_load(WIDE, m) >= 0) OPMX_ISSUE1(LDK, B, g2_load(WIDE, m) >= 0 ? g2_load(WIDE, m) : 0); \
         }                                                                                          \
         wait_vm<(LD2) ? (VM) : 0>();                                                               \
         __builtin_amdgcn_s_barrier();                                                              \
         asm volatile("" ::: "memory");                                                             \
         _Pragma("unroll") for (int m = 0; m < NM; ++m) {                                           \
-            OPMX_MFN(NSB, 1, 1, m);                                                                 \
+            OPMX_MF(1, 1, m);                                                                      \
             if ((NEXT) && m < 4) OPMX_XFRAG((B) ^ 1, 0, 0, m < 4 ? m : 0);                         \
             else if ((NEXT) && m < 4 + TNS) OPMX_WFRAG((B) ^ 1, 0, (m >= 4 && m < 4 + TNS) ? m - 4 : 0); \
         }                                                                                          \
     } while (0)
-#define OPMX_ITER(NSB, KT, B, LD2, NEXT) OPMX_ITERX(NSB, (KT) + 2, B, LD2, NEXT, false, NL)
-    // the k loop of one tile in the form with NSB sub-tiles per wave
-#define OPMX_KLOOP(NSB)                                                                             \
-    do {                                                                                           \
-        int kt = kt0, b = 0;                                                                       \
-        for (; kt + 2 < kt1; ++kt, b ^= 1) OPMX_ITER(NSB, kt, b, true, true);                       \
-        if (kt + 1 < kt1) {                                                                        \
-            OPMX_ITER(NSB, kt, b, false, true);                                                     \
-            ++kt;                                                                                  \
-            b ^= 1;                                                                                \
-        }                                                                                          \
-        OPMX_ITER(NSB, kt, b, false, false);                                                        \
-    } while (0)
+#define OPMX_ITER(KT, B, LD2, NEXT) OPMX_ITERX((KT) + 2, B, LD2, NEXT, false, NL)
 
     // prologue: first k-tile -> buffer 0, second -> buffer 1, wait for the first
 #pragma unroll
@@ -1080,13 +1020,16 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
     for (int i = 0; i < HM; ++i) OPMX_XFRAG(0, 0, 0, i);
 #pragma unroll
     for (int j = 0; j < TNS; ++j) OPMX_WFRAG(0, 0, j);
-    // The k loop and everything behind it, once per form of the tile (NSB sub-tiles per wave).  The
-    // four instances never meet again while accumulators are live: merged behind the k loop, the
-    // accumulators of four paths would have to agree on their registers, and with all 256
-    // accumulation registers in use the register allocator settles that with spills.
-    auto finish_tile = [&](auto nsb_c) __attribute__((always_inline)) {
-    constexpr int NSB = decltype(nsb_c)::value;
-    OPMX_KLOOP(NSB);
+    {
+        int kt = kt0, b = 0;
+        for (; kt + 2 < kt1; ++kt, b ^= 1) OPMX_ITER(kt, b, true, true);
+        if (kt + 1 < kt1) {
+            OPMX_ITER(kt, b, false, true);
+            ++kt;
+            b ^= 1;
+        }
+        OPMX_ITER(kt, b, false, false);
+    }
     // asm MFMAs are opaque to the compiler's hazard padding: let the last ones retire.  The
     // empty statements re-define every accumulator after the wait, so that whatever the register
     // allocator does with a finished accumulator (copy it out, spill it) is placed behind the
@@ -1136,17 +1079,10 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
     }
     // after the last barrier no wave reads operand tiles any more: LDS is free for the epilogue
     if (ncols % 8 == 0 && reinterpret_cast<uintptr_t>(Y) % 16 == 0)
-        tile_epilogue_lds<T, WTM, WTN, SWIGLU, WM>(acc, Bias, Y, mt, N, ncols, n0, wm, wn, lane,
-                                                   smem + wave * (WTM * (SWIGLU ? WTN / 2 : WTN) * 2));
+        tile_epilogue_lds<T, WTM, WTN, SWIGLU>(acc, Bias, Y, mt, N, ncols, n0, wm, wn, lane,
+                                               smem + wave * (WTM * (SWIGLU ? WTN / 2 : WTN) * 2));
     else
-        tile_epilogue<T, WTM, WTN, SWIGLU, WM>(acc, Bias, Y, mt, N, ncols, n0, wm, wn, lane);
-    };
-    switch (nsub) {
-        case 2: finish_tile(std::integral_constant<int, 2>{}); break;
-        case 4: finish_tile(std::integral_constant<int, 4>{}); break;
-        case 6: finish_tile(std::integral_constant<int, 6>{}); break;
-        default: finish_tile(std::integral_constant<int, 8>{}); break;
-    }
+        tile_epilogue<T, WTM, WTN, SWIGLU>(acc, Bias, Y, mt, N, ncols, n0, wm, wn, lane);
 }
 
 __device__ __forceinline__ void store_16(__amdgpu_buffer_rsrc_t r, uint32_t voff, u32x4 v)
@@ -1194,7 +1130,7 @@ __device__ __forceinline__ void load_bias_regs(const T *__restrict__ be, int64_t
         }
 }
 
-template <typename T, int WTM, int WTN, bool SWIGLU, bool BIAS, int ILV>
+template <typename T, int WTM, int WTN, bool SWIGLU, bool BIAS>
 __device__ __forceinline__ void tile_epilogue_staged_impl(
     float4_t (&acc)[WTN / 16][WTM / 16], const T (&bg)[SWIGLU ? WTN / 32 : WTN / 16][4],
     const T (&bu)[SWIGLU ? WTN / 32 : WTN / 16][4], __amdgpu_buffer_rsrc_t ry, int64_t ncols, int64_t nw0, int wm,
@@ -1211,11 +1147,8 @@ __device__ __forceinline__ void tile_epilogue_staged_impl(
     const int c0 = ((lk >> 1) ^ (lrow % CH16)) << 4;
     const int c = lane % CH16, r0 = lane / CH16;
     const int64_t n = nw0 + c * 8;
-    // byte offset of (tile row r0 of the wave's first sub-tile, column n); the next pass is the wave's
-    // next sub-tile: 16 rows further down, or 16 * ILV when the wave rows interleave
-    uint32_t voff = n < ncols ? static_cast<uint32_t>(((wave_subtile_row<WTM, ILV>(wm, 0) + r0) * ncols + n) * 2)
-                              : kDroppedStore;
-    constexpr int SKIP = wave_subtile_row<WTM, ILV>(0, 1) - 16;      // rows of other waves between two passes
+    // byte offset of (tile row wm*WTM + r0, column n); one pass further down is 16 rows
+    uint32_t voff = n < ncols ? static_cast<uint32_t>(((wm * WTM + r0) * ncols + n) * 2) : kDroppedStore;
     const uint32_t row_bytes = static_cast<uint32_t>(ncols * 2);
     u32x4 held[NRD];
 #pragma unroll
@@ -1256,7 +1189,6 @@ __device__ __forceinline__ void tile_epilogue_staged_impl(
                 store_16(ry, voff, held[u]);
                 voff += (n < ncols ? RPI : 0) * row_bytes;
             }
-            if (SKIP > 0) voff += (n < ncols ? SKIP : 0) * row_bytes;
         }
 #pragma unroll
         for (int u = 0; u < NRD; ++u) held[u] = now[u];
@@ -1279,7 +1211,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
                                                                        const T *__restrict__ Bias, int E, int64_t R,
                                                                        int64_t K, int64_t N, T *__restrict__ Y,
                                                                        int ntiles_n, int gnx, int sk_wgs, int sk_cost,
-                                                                       const int32_t *__restrict__ rt, int64_t xrows, int forms)
+                                                                       const int32_t *__restrict__ rt, int64_t xrows)
 {
     constexpr int WM = 2, WN = 2, NW = 4;
     constexpr int WTM = BM / WM, WTN = BN / WN, TMS = WTM / 16, TNS = WTN / 16, HM = TMS / 2;
@@ -1329,10 +1261,11 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
     const int a_lds = wave * LA * 1024, b_lds = BM * ROWB + wave * LB * 1024;
     char *stg = smem + 2 * STAGE + wave * STG;
 
+    float4_t acc[TNS][TMS];            // every tile's first k-tile defines all of them
+
     const int lrow = lane & 15, lk = lane >> 4;
     const int swz = (lrow >> 1) & 7;
-    constexpr int XSTEP = 16 * WM * ROWB;            // interleaved wave rows, as in gemm_tiled_dlds_kernel
-    const int x_off = (wm * 16 + lrow) * ROWB;
+    const int x_off = (wm * WTM + lrow) * ROWB;
     const int w_off = BM * ROWB + (wn * WTN + lrow) * ROWB;
     const int co0 = ((lk ^ swz) << 4), co1 = (((4 + lk) ^ swz) << 4);
     frag xf[2][2][HM], wf[2][TNS];
@@ -1379,60 +1312,35 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
 
         // k-tile 0 overwrites the accumulators.  When k-tile 1 is known to have landed, the NS
         // stores of the previous tile and the 16 loads of this step may still be outstanding.
-        // The k loop in the tile's form (tile_subtiles): all k-tiles but the last two ...
-#define OPMX_KHEAD(NSB)                                                                            \
-    do {                                                                                           \
-        OPMX_ITERX(NSB, 2, b, true, true, true, 16 + NS);                                          \
-        b ^= 1;                                                                                    \
-        for (int kt = 1; kt + 2 < nk; ++kt, b ^= 1) OPMX_ITERX(NSB, kt + 2, b, true, true, false, 16); \
-    } while (0)
-        // ... and the last two, which load the first two k-tiles of the next tile.  Accumulators of
-        // sub-tiles this form leaves out are given a (meaningless) definition here, so that no
-        // accumulator is carried from one tile of the loop to the next; their rows are never stored.
-#define OPMX_KTAIL(NSB)                                                                            \
-    do {                                                                                           \
-        OPMX_ITERX(NSB, 0, b, true, true, false, 16);                                              \
-        b ^= 1;                                                                                    \
-        OPMX_ITERX(NSB, 1, b, true, true, false, 16);                                              \
-        b ^= 1;                                                                                    \
-        _Pragma("unroll") for (int j = 0; j < TNS; ++j)                                            \
-            _Pragma("unroll") for (int i = (NSB); i < TMS; ++i) asm volatile("" : "=a"(acc[j][i])); \
-    } while (0)
-        // One tile in the form with NSB sub-tiles per wave, through to its output stores: the four
-        // instances share no live accumulator (see gemm_tiled_dlds_kernel).
-        auto run_tile = [&](auto nsb_c) __attribute__((always_inline)) {
-            constexpr int NSB = decltype(nsb_c)::value;
-            float4_t acc[TNS][TMS];            // the tile's first k-tile defines the ones this form uses
-            OPMX_KHEAD(NSB);
-            // all loads of this tile are issued: retarget the load state, then stream on
-            rx = x_descriptor(X, nxt.row0, nxt.rows, K, rt, xrows);
-            rw = raw_descriptor(W + static_cast<int64_t>(nxt.e) * N * K);
-            tile_sources<LA, LB, WTN, SWIGLU>(nxt.rows, rt != nullptr, nxt_tok, static_cast<int64_t>(nxt_n) * BNO, K, N, ncols,
-                                              wave, lane, a_src, b_src);
-            const int64_t nw0 = static_cast<int64_t>(cur_n) * BNO + wn * (SWIGLU ? WTN / 2 : WTN);   // first output column of this wave
-            T bg[NOB][4], bu[NOB][4];          // bias of this lane's columns, requested ahead of the last loads
-            if (BIAS) load_bias_regs<T, NOB, SWIGLU>(Bias + static_cast<int64_t>(cur.e) * N, ncols, nw0, lane, bg, bu);
-            OPMX_KTAIL(NSB);
-            // let the last MFMAs retire; re-define the accumulators behind the wait (see
-            // gemm_tiled_dlds_kernel)
-            asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+        OPMX_ITERX(2, b, true, true, true, 16 + NS);
+        b ^= 1;
+        for (int kt = 1; kt + 2 < nk; ++kt, b ^= 1) OPMX_ITERX(kt + 2, b, true, true, false, 16);
+        // all loads of this tile are issued: retarget the load state, then stream on
+        rx = x_descriptor(X, nxt.row0, nxt.rows, K, rt, xrows);
+        rw = raw_descriptor(W + static_cast<int64_t>(nxt.e) * N * K);
+        tile_sources<LA, LB, WTN, SWIGLU>(nxt.rows, rt != nullptr, nxt_tok, static_cast<int64_t>(nxt_n) * BNO, K, N, ncols, wave,
+                                          lane, a_src, b_src);
+        const int64_t nw0 = static_cast<int64_t>(cur_n) * BNO + wn * (SWIGLU ? WTN / 2 : WTN);   // first output column of this wave
+        T bg[NOB][4], bu[NOB][4];          // bias of this lane's columns, requested ahead of the last loads
+        if (BIAS) load_bias_regs<T, NOB, SWIGLU>(Bias + static_cast<int64_t>(cur.e) * N, ncols, nw0, lane, bg, bu);
+        OPMX_ITERX(0, b, true, true, false, 16);
+        b ^= 1;
+        OPMX_ITERX(1, b, true, true, false, 16);
+        b ^= 1;
+        // let the last MFMAs retire; re-define the accumulators behind the wait (see
+        // gemm_tiled_dlds_kernel)
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
-            for (int j = 0; j < TNS; ++j)
+        for (int j = 0; j < TNS; ++j)
 #pragma unroll
-                for (int i = 0; i < TMS; ++i) asm volatile("" : "+a"(acc[j][i]));
+            for (int i = 0; i < TMS; ++i) asm volatile("" : "+a"(acc[j][i]));
+
+        {
             const __amdgpu_buffer_rsrc_t ry =
                 bounded_descriptor(Y + cur.row0 * ncols, static_cast<uint32_t>(cur.rows * ncols * 2));
             // BIAS is a kernel parameter, not a branch: the bias instance needs registers for the
             // lane's bias values, and in one kernel the other path would pay for them with spills
-            tile_epilogue_staged_impl<T, WTM, WTN, SWIGLU, BIAS, WM>(acc, bg, bu, ry, ncols, nw0, wm, lane, stg);
-        };
-        // (with a bias every tile takes the full form: the bias registers and the values that
-        // meet behind four forms do not fit together, and a spill reload drains the pipeline)
-        switch ((BIAS || !forms) ? 8 : tile_subtiles(cur.rows, WM)) {
-            case 2: run_tile(std::integral_constant<int, 2>{}); break;
-            case 4: run_tile(std::integral_constant<int, 4>{}); break;
-            case 6: run_tile(std::integral_constant<int, 6>{}); break;
-            default: run_tile(std::integral_constant<int, 8>{}); break;
+            tile_epilogue_staged_impl<T, WTM, WTN, SWIGLU, BIAS>(acc, bg, bu, ry, ncols, nw0, wm, lane, stg);
         }
         if (!has_next) break;
         cur = nxt;
@@ -1442,13 +1350,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
     // the loads issued for a tile that does not follow must land before the LDS goes away
     wait_vm<0>();
 }
-#undef OPMX_KTAIL
-#undef OPMX_KHEAD
-#undef OPMX_KLOOP
 #undef OPMX_ITER
 #undef OPMX_ITERX
-#undef OPMX_MFN
-#undef OPMX_XFRAGN
 #undef OPMX_MF0
 #undef OPMX_MF
 #undef OPMX_WFRAG
@@ -1529,13 +1432,6 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
     if (option(kOptStreamK) == 0) sk_wgs = 0;    // tuning knob: 0 = off, 2 = split whenever possible
     if (option(kOptStreamK) == 2) sk_cost = 0;
     if (7 * (K / BK) <= 8 * sk_cost) sk_wgs = 0;     // sk_split() cannot split a K this short (g <= 8)
-    // The forms of the k loop for ragged tiles (tile_subtiles) pay while experts hold few row tiles:
-    // a short tile then is a large part of its expert's work.  With many row tiles per expert the
-    // short ones run ahead of the full tiles they share weight tiles with in L2 and the launch as a
-    // whole gets slower (Mixtral shape T=2048 and 64 experts at T=4096: +3 %; T=8192: -1 %; 8x22B
-    // shape at T=4096, four full row tiles and a nearly empty fifth per expert: -4 %).
-    int forms = R / E <= 768 ? 1 : 0;
-    if (option(kOptRagged) >= 0) forms = option(kOptRagged) ? 1 : 0;      // tuning knob
     int *sk_count = static_cast<int *>(ws);
     float *sk_part = reinterpret_cast<float *>(static_cast<char *>(ws) + kSkCounters * sizeof(int));
     dim3 grid(static_cast<unsigned>(dp_ids));
@@ -1568,7 +1464,7 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
         static std::atomic<uint64_t> attr_p[4];
         const bool hb = B != nullptr;
         using kernel_t = void (*)(const T *, const int64_t *, const T *, const T *, int, int64_t, int64_t, int64_t, T *, int,
-                                  int, int, int, const int32_t *, int64_t, int);
+                                  int, int, int, const int32_t *, int64_t);
         const kernel_t kp = sw ? (hb ? gemm_tiled_dlds_persist_kernel<T, BM, BN, true, true>
                                      : gemm_tiled_dlds_persist_kernel<T, BM, BN, true, false>)
                                : (hb ? gemm_tiled_dlds_persist_kernel<T, BM, BN, false, true>
@@ -1578,14 +1474,14 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
         // ids congruent mod 8 stay on one XCD as long as the grid is a multiple of 8
         const unsigned wgs = static_cast<unsigned>(dp_ids < cus ? dp_ids : cus);
         if (sk_wgs > 0) sk_clear_kernel<<<1, 256, 0, s>>>(sk_count, kSkCounters);
-        kp<<<wgs, block, smem_p, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n, gnx, sk_wgs, sk_cost, g.index, g.x_rows, forms);
+        kp<<<wgs, block, smem_p, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n, gnx, sk_wgs, sk_cost, g.index, g.x_rows);
         if (sk_wgs > 0) {
             if (sw)
                 gemm_tiled_dlds_kernel<T, BM, BN, true, true><<<sk_wgs, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
-                                                                                          gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows, forms);
+                                                                                          gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows);
             else
                 gemm_tiled_dlds_kernel<T, BM, BN, false, true><<<sk_wgs, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
-                                                                                           gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows, forms);
+                                                                                           gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows);
         }
         OPMX_LAUNCH_CHECK();
         return OPMX_OK;
@@ -1593,16 +1489,16 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
     if (sk_wgs > 0) sk_clear_kernel<<<1, 256, 0, s>>>(sk_count, kSkCounters);
     if (sw) {
         gemm_tiled_dlds_kernel<T, BM, BN, true, false><<<grid, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
-                                                                                 gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows, forms);
+                                                                                 gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows);
         if (sk_wgs > 0)
             gemm_tiled_dlds_kernel<T, BM, BN, true, true><<<sk_wgs, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
-                                                                                      gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows, forms);
+                                                                                      gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows);
     } else {
         gemm_tiled_dlds_kernel<T, BM, BN, false, false><<<grid, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
-                                                                                  gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows, forms);
+                                                                                  gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows);
         if (sk_wgs > 0)
             gemm_tiled_dlds_kernel<T, BM, BN, false, true><<<sk_wgs, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
-                                                                                       gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows, forms);
+                                                                                       gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows);
     }
     OPMX_LAUNCH_CHECK();
     return OPMX_OK;
