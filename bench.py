@@ -24,9 +24,10 @@ already resident in HBM.  Prints ONE JSON line:
   vendor_dense_gemm_same_flops_TFLOPs
                        MFMA-bound workloads: the vendor library's dense GEMM with the flop
                        count of the gate/up launch (no expert grouping), context only
-  companion            with the default workload: every other configuration of the benchmark set
-                       (decode T=1/8/128, T=512/1024, prefill T=2048/8192, 64 experts T=32/4096,
-                       8x22B shape T=16/4096), each measured by a child process of this program
+  companion            with the default workload: every configuration of the benchmark set
+                       (decode T=1/8/32/128, T=512/1024, prefill T=2048/8192, 64 experts T=32/4096,
+                       8x22B shape T=16/4096), each as the operator-by-operator sequence and with the
+                       fused forms (--fused), measured by child processes of this program
   cpu_baseline         the CPU oracle (PyTorch CPU restatement of the reference
                        operator sequence) on the host cores, bounded sample
 
@@ -91,10 +92,12 @@ def measured_traffic(workload, fused):
     return None, stale or "no counter run for this workload under profiles/"
 
 
-# configurations of the benchmark set measured beside the default workload (child processes)
-COMPANIONS = [("decode-T1", []), ("decode-T8", []), ("decode-T128", []), ("decode-T512", []), ("decode-T1024", []),
-              ("prefill-T2048", []), ("prefill-T8192", []), ("prefill-T8192", ["--fuse-swiglu"]),
-              ("fine-T32", []), ("fine-T4096", []), ("8x22b-T16", []), ("8x22b-T4096", [])]
+# configurations of the benchmark set measured beside the default workload (child processes), each as
+# the operator-by-operator sequence and with the fused forms MoeFeedForward uses by default
+COMPANIONS = [(w, f) for w in ("decode-T1", "decode-T8", "decode-T32", "decode-T128", "decode-T512", "decode-T1024",
+                               "prefill-T2048", "prefill-T8192", "fine-T32", "fine-T4096", "8x22b-T16", "8x22b-T4096")
+              for f in ([], ["--fused"]) if not (w == "decode-T32" and not f)]
+
 
 SHAPES = {
     "decode": dict(H=4096, E=8, k=2, I=14336, dtype="float16", skew=0.0, name="mixtral-8x7b"),
@@ -150,7 +153,12 @@ def main():
                          "the reference reading for FETCH_SIZE / WRITE_SIZE counter runs")
     ap.add_argument("--kernel-sources-hash", action="store_true",
                     help="print the hash that a bench-traffic line under profiles/ must carry for this tree, and exit")
+    ap.add_argument("--fused", action="store_true",
+                    help="all three fused forms (--fuse-swiglu --fuse-gather --fuse-router-select): the block as "
+                         "MoeFeedForward runs it by default")
     args = ap.parse_args()
+    if args.fused:
+        args.fuse_swiglu = args.fuse_gather = args.fuse_router_select = True
     if args.kernel_sources_hash:
         print(kernel_sources_sha256())
         return
@@ -180,13 +188,13 @@ def main():
         import subprocess
         companion = {}
         for name, extra in COMPANIONS:
-            cmd = [sys.executable, os.path.abspath(__file__), "--workload", name, "--steps", "50", "--warmup", "5",
-                   "--windows", "2", "--no-cpu-baseline", "--no-device-ceilings", "--no-vendor-gemm",
-                   "--no-companion"] + extra
+            cmd = [sys.executable, os.path.abspath(__file__), "--workload", name, "--steps", "40", "--warmup", "5",
+                   "--windows", "2", "--conditioning-ms", "200", "--no-cpu-baseline", "--no-device-ceilings",
+                   "--no-vendor-gemm", "--no-companion"] + extra
             try:
                 line = subprocess.run(cmd, capture_output=True, text=True, timeout=300, check=True).stdout.strip().splitlines()[-1]
                 r = json.loads(line)
-                companion[name + (", fused SwiGLU epilogue" if extra else "")] = {
+                companion[name + (", fused forms" if extra else "")] = {
                     key: r[key] for key in ("value", "unit", "ms_per_step", "steps", "windows", "config", "roofline",
                                             "layer", "hip_graph_replay", "per_op_us")}
             except Exception as exc:

@@ -27,6 +27,11 @@ class MoeFeedForward(nn.Module):
     """``args`` needs ``hidden_dim, intermediate_dim, num_experts, num_experts_per_token``
     (the fields of the reference's ``ModelParams`` this block reads).
 
+    The block computes what the reference's operator sequence computes and, by default, runs it
+    through the three fused forms below (all flags ``False``: one launch sequence per reference
+    operator, the form ``bench.py`` reports as its headline value; ONNX export always takes the
+    operator-by-operator route, so the exported graph is the reference's either way).
+
     ``fuse_swiglu_epilogue=True`` (only with ``fused_ffn_glu``) applies SwiGLU
     inside the gate/up GEMM instead of as a separate operator; results agree
     to rounding, the ONNX graph does not change because export always takes
@@ -40,8 +45,8 @@ class MoeFeedForward(nn.Module):
     """
 
     def __init__(self, args, layer_id: int, fused_ffn_glu: bool, linear_bias_term: bool, proc_group,
-                 dtype=None, device=None, fuse_swiglu_epilogue: bool = False, fuse_router_select: bool = False,
-                 fuse_x_gather: bool = False):
+                 dtype=None, device=None, fuse_swiglu_epilogue: bool = True, fuse_router_select: bool = True,
+                 fuse_x_gather: bool = True):
         super().__init__()
         self.fuse_x_gather = fuse_x_gather
         self.layer_id = layer_id
@@ -201,8 +206,8 @@ class GraphedMoeFeedForward(nn.Module):
 
 
 def load_opmx_moe_block(path, layer_id: int, num_experts_per_token: int, fused_ffn_glu: bool = True,
-                        dtype=None, device=None, fuse_swiglu_epilogue: bool = False, fuse_router_select: bool = False,
-                        fuse_x_gather: bool = False):
+                        dtype=None, device=None, fuse_swiglu_epilogue: bool = True, fuse_router_select: bool = True,
+                        fuse_x_gather: bool = True):
     """Builds the MoE block of layer ``layer_id`` from an OPMX Mixtral ``.pth`` checkpoint.
 
     The file is opened with ``weights_only=True`` and memory-mapped, so only this layer's tensors are

@@ -16,17 +16,21 @@ from test_gpu_layer import build_layer
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("T,H,I,E,k,dtype,fuse,route", [
-    (1, 1024, 2816, 8, 2, torch.float16, False, False),    # single token: 16-row stream kernel, small select
-    (32, 1024, 2816, 8, 2, torch.float16, True, False),    # stream kernel with the SwiGLU epilogue
-    (8, 1024, 2816, 8, 2, torch.float16, True, True),      # ... and router gate + select in one launch
-    (40, 512, 1408, 64, 8, torch.bfloat16, False, False),  # 64 experts, short K
-    (256, 1024, 3584, 8, 2, torch.float16, False, False),  # 128 x 256 tiles, down projection split over K
-    (3000, 512, 1024, 8, 2, torch.float16, False, True),   # large select path, persistent 256 x 256 tiles
+@pytest.mark.parametrize("T,H,I,E,k,dtype,fuse,route,gather", [
+    (1, 1024, 2816, 8, 2, torch.float16, False, False, False),    # single token: 16-row stream kernel, small select
+    (32, 1024, 2816, 8, 2, torch.float16, True, False, False),    # stream kernel with the SwiGLU epilogue
+    (8, 1024, 2816, 8, 2, torch.float16, True, True, False),      # ... and router gate + select in one launch
+    (8, 1024, 2816, 8, 2, torch.float16, True, True, True),       # ... and the rows read through the index
+    (40, 512, 1408, 64, 8, torch.bfloat16, False, False, False),  # 64 experts, short K
+    (256, 1024, 3584, 8, 2, torch.float16, False, False, False),  # 128 x 256 tiles, down projection split over K
+    (3000, 512, 1024, 8, 2, torch.float16, False, True, False),   # large select path, persistent 256 x 256 tiles
+    (5000, 512, 1024, 8, 2, torch.float16, True, True, True),     # every fused form: routing in the router kernel's
+                                                                  # epilogue, rows through the index, persistent tiles
+    (700, 512, 1408, 64, 8, torch.bfloat16, True, True, True),    # the same with 64 experts
 ])
-def test_captured_layer_replays_the_eager_result(T, H, I, E, k, dtype, fuse, route):
+def test_captured_layer_replays_the_eager_result(T, H, I, E, k, dtype, fuse, route, gather):
     (x, Wg, wu, w2), _ = gpu_inputs(T, H, E, I, dtype, seed=3)
-    layer = build_layer(H, I, E, k, dtype, Wg, wu, w2, fuse=fuse, route=route)
+    layer = build_layer(H, I, E, k, dtype, Wg, wu, w2, fuse=fuse, route=route, gather=gather)
     gen = torch.Generator(device="cuda").manual_seed(11)
     inputs = [x] + [torch.randn(T, H, generator=gen, device=dev()).to(dtype) for _ in range(3)]
     with torch.inference_mode():

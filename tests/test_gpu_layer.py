@@ -14,10 +14,11 @@ pytestmark = pytest.mark.gpu
 MAX_ABS, MEAN_ABS = 2e-2, 2e-3
 
 
-def build_layer(H, I, E, k, dtype, Wg, wu, w2, fuse=False, route=False):
+def build_layer(H, I, E, k, dtype, Wg, wu, w2, fuse=False, route=False, gather=False):
+    """The block with the fused forms named (none: one launch sequence per reference operator)."""
     from model_zoo.mixtral.modeling.dynamic_batching.Model import MoeFeedForward
     m = MoeFeedForward(MoeFeedForward.params(H, I, E, k), 0, True, False, None, dtype=dtype, device=dev(),
-                       fuse_swiglu_epilogue=fuse, fuse_router_select=route)
+                       fuse_swiglu_epilogue=fuse, fuse_router_select=route, fuse_x_gather=gather)
     m.gate.weight.data = Wg
     m.wu.weight.data = wu
     m.w2.weight.data = w2
@@ -116,8 +117,8 @@ def test_mixtral_8x7b_decode(mixtral_8x7b, T):
     check_against_oracle(gr, (host[0][:T],) + host[1:], 8, 2)
     mr = build_layer(4096, 14336, 8, 2, torch.float16, Wg, wu, w2, route=True)
     assert torch.equal(mr(x[:T]), gr["out"])
-    # both fused forms together, against the oracle routed by the fused call's logits
-    mfr = build_layer(4096, 14336, 8, 2, torch.float16, Wg, wu, w2, fuse=True, route=True)
+    # all fused forms together (the block's default), against the oracle routed by the fused call's logits
+    mfr = build_layer(4096, 14336, 8, 2, torch.float16, Wg, wu, w2, fuse=True, route=True, gather=True)
     check_fused_against_oracle(mfr(x[:T]), gr, (host[0][:T],) + host[1:], 8, 2)
 
 
@@ -130,8 +131,8 @@ def test_mixtral_8x7b_prefill_skewed(mixtral_8x7b, T, full):
     counts = (g["off"][1:] - g["off"][:-1]).cpu()
     assert float(counts.max()) / (T * k) > 0.40, counts.tolist()
     check_against_oracle(g, (host[0][:T],) + host[1:], E, k, bias=bias, full=full)
-    for route in (False, True):     # SwiGLU in the GEMM epilogue, alone and with the fused router call
-        mf = build_layer(4096, 14336, E, k, torch.float16, Wg, wu, w2, fuse=True, route=route)
+    for route in (False, True):     # SwiGLU in the GEMM epilogue alone, and all fused forms (the block's default)
+        mf = build_layer(4096, 14336, E, k, torch.float16, Wg, wu, w2, fuse=True, route=route, gather=route)
         mf.gate.bias = torch.nn.Parameter(bias.to(dev()), requires_grad=False)
         check_fused_against_oracle(mf(x[:T]), g, (host[0][:T],) + host[1:], E, k, full=full)
     # size-independent property: the layer is row-wise, so a row subset gives the same rows
@@ -148,7 +149,7 @@ def test_fine_grained_64_experts_bf16(T):
     g = run_ops(x, Wg, wu, w2, E, k)
     check_against_oracle(g, host, E, k)
     for route in (False, True):
-        mf = build_layer(H, I, E, k, torch.bfloat16, Wg, wu, w2, fuse=True, route=route)
+        mf = build_layer(H, I, E, k, torch.bfloat16, Wg, wu, w2, fuse=True, route=route, gather=route)
         check_fused_against_oracle(mf(x), g, host, E, k)
 
 
@@ -158,5 +159,5 @@ def test_mixtral_8x22b_shape(T, full):
     (x, Wg, wu, w2), host = gpu_inputs(T, H, E, I, torch.float16, seed=4)
     g = run_ops(x, Wg, wu, w2, E, k)
     check_against_oracle(g, host, E, k, full=full)
-    mf = build_layer(H, I, E, k, torch.float16, Wg, wu, w2, fuse=True)
+    mf = build_layer(H, I, E, k, torch.float16, Wg, wu, w2, fuse=True, route=T > 8, gather=True)
     check_fused_against_oracle(mf(x), g, host, E, k, full=full)
