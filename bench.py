@@ -58,7 +58,8 @@ MFMA_PEAK_TFLOPS = 2500.0      # dense fp16/bf16 MFMA, vendor figure
 # HBM bytes per launch of the dominant kernel come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # of this program, each scaled by the same counter's reading for a plain copy kernel of known size.
 # The summaries under profiles/ record them in a line
-#   bench-traffic: workload=<name> fused_swiglu=<0|1> bytes_per_launch=<n> kernel_sources_sha256=<hex>
+#   bench-traffic: workload=<name> forms=<none|swiglu|all> bytes_per_launch=<n> kernel_sources_sha256=<hex>
+# (forms: which fused forms the run used: none, the SwiGLU epilogue alone, or all three as with --fused)
 # together with the hash of the kernel sources the counter run was made with; a line whose hash
 # is not that of the sources in this tree is out of date and is not reported.
 def kernel_sources_sha256():
@@ -74,16 +75,16 @@ def kernel_sources_sha256():
     return h.hexdigest()
 
 
-def measured_traffic(workload, fused):
+def measured_traffic(workload, forms):
     """(bytes per launch or None, where the figure comes from / why there is none)."""
     import glob
     import re
     want = kernel_sources_sha256()
     stale = None
     for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.txt"))):
-        for m in re.finditer(r"bench-traffic: workload=(\S+) fused_swiglu=([01]) bytes_per_launch=(\d+) "
+        for m in re.finditer(r"bench-traffic: workload=(\S+) forms=(\w+) bytes_per_launch=(\d+) "
                              r"kernel_sources_sha256=([0-9a-f]+)", open(path).read()):
-            if m.group(1) != workload or bool(int(m.group(2))) != bool(fused):
+            if m.group(1) != workload or m.group(2) != forms:
                 continue
             rel = os.path.relpath(path, ROOT)
             if m.group(4) == want:
@@ -409,7 +410,9 @@ def main():
     gemm1_flops = 2.0 * R * H * 2 * I
     layer_bytes = w_bytes_gemm1 + w_bytes_gemm2 + 2 * T * H * s + E * H * s
     layer_flops = T * (k * (2.0 * H * 2 * I + 2.0 * I * H) + 2.0 * H * E)
-    traffic, traffic_source = measured_traffic(args.workload, args.fuse_swiglu)
+    fl = (args.fuse_swiglu, args.fuse_gather, args.fuse_router_select)
+    forms = {(False, False, False): "none", (True, False, False): "swiglu", (True, True, True): "all"}.get(fl, "other")
+    traffic, traffic_source = measured_traffic(args.workload, forms)
     hbm_bound = (layer_flops / layer_bytes) < (MFMA_PEAK_TFLOPS * 1e12) / (HBM_PEAK_GBS * 1e9)
     if hbm_bound:
         ach = gemm1_bytes / (gemm1_ms * 1e-3) / 1e9
