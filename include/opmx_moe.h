@@ -81,7 +81,7 @@ const char *opmx_status_string(int status);
  *   "OPMX_MOE_GEMM_TILED_VARIANT"  0 256x256 direct-to-LDS, 1 256x256 register-staged,
  *                                  2 128x128 register-staged, 3 128x256 direct-to-LDS
  *   "OPMX_MOE_GEMM_STREAM_VARIANT" 0..5: chunk widths / prefetch depth of the streaming kernel
- *   "OPMX_MOE_GEMM_GNX"            tile order: 8 expert-major, 16 row partition, 4, 0 row-major
+ *   "OPMX_MOE_GEMM_GNX"            tile order: 8 expert-major, 16 row partition, 32 expert-grouped, 4, 0 row-major
  *   "OPMX_MOE_GEMM_STREAMK"        0 never split the tail tiles over K, 2 whenever possible
  *   "OPMX_MOE_GEMM_PERSIST"        0 never the persistent form, 1 whenever its conditions hold
  * Returns OPMX_ERR_BAD_ARGUMENT for an unknown name. */

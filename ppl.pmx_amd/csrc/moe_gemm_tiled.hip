@@ -262,13 +262,54 @@ __device__ __forceinline__ void map_row_partition(int64_t lin, int mtiles, int n
     tile_n = static_cast<int>(c);
 }
 
+// Expert-grouped partition (gnx = 32), for many small experts (a few row tiles each).  All tiles
+// are strung together expert by expert and, inside an expert, in row groups of up to 8 row tiles:
+// for each group, for each column tile, the rows of the group.  XCD x (ids = x mod 8) owns the
+// contiguous eighth [x*ttot/8, (x+1)*ttot/8) of that string, so its 32 resident workgroups cover
+// all m row tiles of one expert times 32/m column tiles: every W-tile is shared by all rows of its
+// expert and fetched by one XCD, the expert's X rows by that XCD alone, and the XCDs are balanced to
+// one tile.  (The expert-major order gives every XCD an eighth of every expert: with two or three
+// row tiles per expert an XCD's workgroups then sit in a dozen experts at once and every XCD
+// fetches every X row.)  Up to 7 ids past the end name no tile.  Grouped launches only.
+__device__ __forceinline__ void locate_expert_grouped(int64_t lin, const ExpertTable &tab, int BM, int mtiles, int ntiles_n,
+                                                      MTile &mt, int &tile_n)
+{
+    mt.e = 0;
+    mt.rows = 0;
+    mt.row0 = 0;
+    tile_n = 0;
+    const uint64_t ttot = static_cast<uint64_t>(mtiles) * static_cast<uint32_t>(ntiles_n);
+    const uint32_t xcd = static_cast<uint32_t>(lin) & 7;
+    const uint64_t j = static_cast<uint64_t>(lin) >> 3, lo = xcd * ttot / 8, hi = (xcd + 1) * ttot / 8;
+    if (lin < 0 || j >= hi - lo) return;
+    const uint32_t g = static_cast<uint32_t>(lo + j), nt = static_cast<uint32_t>(ntiles_n);
+    const int e = find_expert(static_cast<int>(g / nt), tab);
+    if (e < 0) return;
+    const uint32_t first = static_cast<uint32_t>(tab.pref[e]), m = static_cast<uint32_t>(tab.pref[e + 1]) - first;
+    const uint32_t l = g - first * nt, per_group = 8 * nt, full = m >> 3;
+    uint32_t rg = l / per_group, h = 8;
+    if (rg >= full) {
+        rg = full;
+        h = m - 8 * full;
+    }
+    const uint32_t t = l - rg * per_group, c = t / h, row = rg * 8 + (t - c * h);
+    const int64_t row0 = tab.off[e] + static_cast<int64_t>(row) * BM, left = tab.off[e + 1] - row0;
+    tile_n = __builtin_amdgcn_readfirstlane(static_cast<int>(c));
+    mt.e = __builtin_amdgcn_readfirstlane(e);
+    mt.row0 = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0 >> 32))) << 32) |
+              static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row0)));
+    mt.rows = __builtin_amdgcn_readfirstlane(static_cast<int>(left < BM ? left : BM));
+}
+
 // Linear tile id -> tile, in whichever order gnx names.  mt.rows == 0: the id names no work.
 __device__ __forceinline__ void locate_any(int64_t lin, int gnx, int mtiles, int ntiles_n, bool grouped,
                                            const ExpertTable &s_off, int E, int64_t R, int BM, MTile &mt, int &tile_n)
 {
     if (gnx == 8) {
         locate_expert_major(lin, grouped, s_off, E, R, BM, ntiles_n, mt, tile_n);
-    } else if (gnx == 16) {
+    } else if (gnx == 32 && grouped) {
+        locate_expert_grouped(lin, s_off, BM, mtiles, ntiles_n, mt, tile_n);
+    } else if (gnx == 16 || gnx == 32) {
         int tile_m;
         map_row_partition(lin, mtiles, ntiles_n, tile_m, tile_n);
         if (tile_m >= mtiles || tile_n >= ntiles_n) tile_m = -1;
@@ -282,12 +323,15 @@ __device__ __forceinline__ void locate_any(int64_t lin, int gnx, int mtiles, int
 }
 
 // Host side of map_tile: the order to use and the number of linear ids it spans.
-inline int pick_gnx(int ntiles_n)
+// small_experts: a grouped launch whose experts hold a few row tiles each on average.
+inline int pick_gnx(int ntiles_n, bool grouped = false, bool small_experts = false)
 {
     // XCD-grouped orders only when the n-tiles split evenly over the XCDs (else XCDs idle)
     int gnx = ntiles_n % 8 == 0 ? 8 : 16;
+    if (grouped && small_experts) gnx = 32;
     if (option(kOptGnx) >= 0) gnx = option(kOptGnx);   // tuning knob
-    if (gnx != 0 && gnx != 4 && gnx != 8 && gnx != 16) gnx = 0;
+    if (gnx == 32 && !grouped) gnx = ntiles_n % 8 == 0 ? 8 : 16;
+    if (gnx != 0 && gnx != 4 && gnx != 8 && gnx != 16 && gnx != 32) gnx = 0;
     if (gnx == 4 && ntiles_n % 16 != 0) gnx = 0;
     if (gnx == 8 && ntiles_n % 8 != 0) gnx = 0;
     return gnx;
@@ -296,6 +340,7 @@ inline int64_t linear_ids(int gnx, int ntiles_m, int ntiles_n)
 {
     if (gnx == 8) return static_cast<int64_t>(ntiles_n) * ntiles_m;     // exactly the tiles
     if (gnx == 16) return 8 * ceil_div(ntiles_m, 8) * ntiles_n;          // every XCD as long as the longest
+    if (gnx == 32) return 8 * ceil_div(static_cast<int64_t>(ntiles_n) * ntiles_m, 8);
     if (gnx == 4) return ceil_div(ntiles_n, 16) * ceil_div(ntiles_m, 16) * 256;
     return static_cast<int64_t>(ntiles_n) * ntiles_m;
 }
@@ -1241,7 +1286,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
     // ids [nmain, ttot) are the tail launch's.  The row-partition order has ids that name no tile
     // behind the last tile of each XCD: its id space is longer than the tile count, and a
     // workgroup's stream ends at the first such id (all later ones of its XCD are empty too).
-    const int64_t ids = gnx == 16 ? int64_t{8} * ((mtiles + 7) / 8) * ntiles_n : ttot;
+    const int64_t ids = gnx == 16 ? int64_t{8} * ((mtiles + 7) / 8) * ntiles_n : (gnx == 32 ? (ttot + 7) / 8 * 8 : ttot);
     const int64_t nmain = g > 1 ? ttot - ttot % sk_wgs : ids;
     int64_t id = blockIdx.x;
     if (id >= nmain) return;
@@ -1416,7 +1461,14 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
     const int64_t ncols = sw ? N / 2 : N;
     const int ntiles_n = static_cast<int>(ceil_div(ncols, sw ? BN / 2 : BN));
     const int ntiles_m = static_cast<int>(max_mtiles(R, E, BM));
-    const int gnx = pick_gnx(ntiles_n);
+    // Many small experts -- on average up to 96 tiles each, three times what an XCD holds at a time --
+    // and no tail split: expert-grouped order.  Measured against the expert-major / row-partition
+    // orders: 64 experts x (2-3 row tiles x 11 or 8 column tiles) -11 % and -12 % time, 4-5 row tiles
+    // -3 % and -3 %, 8-9 row tiles +1 % and -5 %; 128 experts x (4-5 x 6 or 8) -5 % and -4 %; experts of
+    // 170 tiles and more +6 ... +14 % (an XCD alone on an expert re-reads its X rows for every handful
+    // of columns, and no other XCD has brought them into the memory-side cache).
+    const bool small_experts = off != nullptr && K / BK <= 128 && (2 * R + int64_t{E} * BM) * ntiles_n <= int64_t{192} * E * BM;
+    const int gnx = pick_gnx(ntiles_n, off != nullptr, small_experts);
     const int64_t dp_ids = linear_ids(gnx, ntiles_m, ntiles_n);
     if (dp_ids >= (int64_t{1} << 31)) return OPMX_ERR_UNSUPPORTED;
     // split-K of the tail tiles when the caller lends the scratch memory for it.  The tile count
@@ -1452,7 +1504,7 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
     // short enough for the tile switch to matter.  Measured: +3-12 % up to K = 4096, even at
     // 8192, -2 % at K = 14336, where the fixed pairing of workgroups and tiles lets the
     // workgroups of an XCD drift apart over the rounds and share less in L2 (+13 % HBM reads).
-    bool persist = (gnx == 4 || gnx == 8 || gnx == 16) && K / BK >= 4 && ncols % 8 == 0 && reinterpret_cast<uintptr_t>(Y) % 16 == 0 &&
+    bool persist = (gnx == 4 || gnx == 8 || gnx == 16 || gnx == 32) && K / BK >= 4 && ncols % 8 == 0 && reinterpret_cast<uintptr_t>(Y) % 16 == 0 &&
                    ncols * (2 * BM) < (int64_t{1} << 31) && cus >= 8 && cus % 8 == 0;
     if (option(kOptPersist) >= 0) {              // tuning knob: 0 = never, 1 = whenever possible
         if (option(kOptPersist) == 0) persist = false;

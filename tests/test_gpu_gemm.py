@@ -121,6 +121,31 @@ def test_expert_major_and_row_partition_tile_orders(variant):
     run_case("column", [70] * 19, 64, 2816, torch.float16, False, env, swiglu=True)   # 19 row tiles, 11 column tiles of 128
 
 
+@pytest.mark.parametrize("variant", ["0", "3"])
+def test_expert_grouped_tile_order(variant):
+    """The order for many small experts (each XCD owns a contiguous eighth of the tiles strung
+    together expert by expert): chosen by itself up to four row tiles per expert on average,
+    forced here for experts with more than one row group of 8 as well.  Tile counts that are and
+    are not multiples of 8, fewer tiles than XCDs, empty experts, 11 and 8 column tiles, the
+    persistent form walking several tiles per workgroup; same bits as the expert-major order."""
+    env = {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": variant, "OPMX_MOE_GEMM_GNX": "32"}
+    g = torch.Generator().manual_seed(7)
+    small = [int(v) for v in torch.randint(480, 545, (64,), generator=g)]      # two or three row tiles of 256 each
+    small[5] = small[40] = 0
+    a = run_case("column", small, 128, 2816, torch.bfloat16, False, env)          # 11 column tiles
+    b = run_case("column", small, 128, 2816, torch.bfloat16, False, dict(env, OPMX_MOE_GEMM_GNX="16"))
+    assert torch.equal(a, b)
+    a = run_case("row", small, 192, 2048, torch.float16, True, env)               # 8 column tiles
+    b = run_case("row", small, 192, 2048, torch.float16, True, dict(env, OPMX_MOE_GEMM_GNX="8"))
+    assert torch.equal(a, b)
+    run_case("column", small, 64, 4096, torch.float16, True, env, swiglu=True)
+    run_case("column", [4200, 0, 300, 5000, 17, 256, 1, 2100], 128, 2048, torch.float16, True, env)   # row groups of 8 + rest
+    run_case("row", [3], 64, 256, torch.float16, False, env)                      # one tile
+    run_case("row", [300, 0, 129], 128, 768, torch.bfloat16, False, env)          # 9 (variant 3: 15) tiles
+    # what the library picks by itself for this shape
+    run_case("column", small, 128, 2816, torch.bfloat16, False, {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": variant})
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_persistent_kernel_streams_tiles(dtype):
     """The persistent form of the 256x256 kernel (16 column tiles, K >= 256): fewer tiles than
