@@ -299,9 +299,12 @@ int stream_swiglu_impl(const void *X, const int64_t *off, const void *W, const v
                        int64_t N, int64_t rows_hint, void *Y, hipStream_t s, RowGather g)
 {
     const int64_t m = rows_hint > 0 ? rows_hint : R;
-    if (m <= 2)      // short K: narrower chunks, as in stream_pick_mt
+    if (m <= 2) {    // short K: narrower chunks, as in stream_pick_mt
+        if (K >= 16 * 256 && ceil_div(N / 2, 64) * (R < E ? R : E) >= 256)
+            return stream_launch_sw<T, 1, 256, 2, true, 4, false, false, true>(X, off, W, B, E, R, K, N, Y, s, g);
         return K < 16 * 256 ? stream_launch<T, 1, 128, 2, true, true>(X, off, W, B, E, R, K, N, Y, s, g)
                             : stream_launch<T, 1, 256, 2, true, true>(X, off, W, B, E, R, K, N, Y, s, g);
+    }
     if (m <= 32) {
         // long K: SwiGLU by wave pairs, which keeps the plain form's 256-wide chunks and LDS footprint
         // (a wave with two row groups needs twice the strip: chunks half as wide, or half the waves
