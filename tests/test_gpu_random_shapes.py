@@ -95,8 +95,11 @@ def test_layer_random(seed):
     check_against_oracle(g, host, E, k)
     gr = run_ops(x, Wg, wu, w2, E, k, route=True)
     check_against_oracle(gr, host, E, k)
-    for fuse, route in ((True, False), (True, True)):
-        m = build_layer(H, I, E, k, dtype, Wg, wu, w2, fuse=fuse, route=route)
+    for fuse, route, gather in ((True, False, False), (True, True, False), (False, False, True), (True, True, True)):
+        m = build_layer(H, I, E, k, dtype, Wg, wu, w2, fuse=fuse, route=route, gather=gather)
         want = gr["out"] if route else g["out"]
+        if not fuse:           # the gather alone changes no bit
+            assert torch.equal(m(x), want)
+            continue
         err = (m(x).double() - want.double()).abs()
-        assert float(err.max()) <= 2e-2 and float(err.mean()) <= 2e-3, (fuse, route, float(err.max()))
+        assert float(err.max()) <= 2e-2 and float(err.mean()) <= 2e-3, (fuse, route, gather, float(err.max()))
