@@ -33,7 +33,11 @@ template <bool NT> __device__ __forceinline__ u32x4 ld16(const char *p)
     return *reinterpret_cast<const u32x4 *>(p);
 }
 
-template <typename T, int MT, int KC, int DEPTH, bool NT, int SW, bool SG, bool PAIR, bool SGW = false>
+// XR: X rows a tile holds and the block stages per K chunk.  16*MT normally; 2 for calls with at most two rows
+// in all (a single token with two experts): the MFMA still multiplies 16 columns, the lanes of the
+// fourteen that do not exist read the last staged row again, and the X chunk is 1 KiB instead of 8 --
+// with one row per expert the sixteen-row staging moved as many bytes through LDS as the weights.
+template <typename T, int MT, int KC, int DEPTH, bool NT, int SW, bool SG, bool PAIR, bool SGW = false, int XR = 16 * MT>
 __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restrict__ X,
                                                                const int64_t *__restrict__ off,
                                                                const T *__restrict__ W,
@@ -54,12 +58,14 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
     constexpr int RS = KC * 2 + 16;              // LDS row stride in bytes (pad 16: conflict-free strips)
     constexpr int RPL = 512 / KC;                // W rows covered by one wave load (1 KiB)
     constexpr int NLW = 16 / RPL;                // W loads per wave per chunk
-    constexpr int XM = 16 * MT;                  // X rows per tile
+    constexpr int XM = XR;                       // X rows per tile
     constexpr int CPR = KC / 8;                  // 16-byte chunks per row per K-chunk
-    constexpr int NLX = XM * CPR / (SW * 64);    // X loads per thread per chunk
+    constexpr bool XW0 = XM * CPR == 64 && SW > 1;                   // the X chunk is one wave load: every wave makes it
+    constexpr int NLX = XW0 ? 1 : XM * CPR / (SW * 64);              // X loads per thread per chunk
     constexpr int WSTRIP = NG * 16 * RS;
     constexpr int XBUF = XM * RS;
-    static_assert(XM * CPR % (SW * 64) == 0, "X chunk must divide over the block");
+    static_assert(XW0 || XM * CPR % (SW * 64) == 0, "X chunk must divide over the block");
+    static_assert(XR == 16 * MT || (MT == 1 && XR < 16), "short tiles: one MFMA tile of rows");
     static_assert(DEPTH == 1 || DEPTH == 2, "one or two chunks in flight");
     using frag = typename Mfma<T>::frag;
 
@@ -98,7 +104,9 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
     int xdst[NLX], xk[NLX];
 #pragma unroll
     for (int i = 0; i < NLX; ++i) {
-        const int q = tid + SW * 64 * i, row = q / CPR, c = q % CPR;
+        // XW0: all waves load and stage the same 1 KiB (identical bytes to identical places: a branch that
+        // left it to one wave would cost the others their load pipelining, the compiler then waits for everything)
+        const int q = XW0 ? lane : tid + SW * 64 * i, row = q / CPR, c = q % CPR;
         const int r = row < mt.rows ? row : mt.rows - 1;
         xrow[i] = static_cast<uint32_t>((rt ? gathered_row(rt, xrows, mt.row0 + r) : r) * K * 2);
         xdst[i] = row * RS + c * 16;
@@ -152,6 +160,7 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
     } while (0)
 
     const int fr = lane & 15, fg = lane >> 4;   // fragment row (W row / X row) and k group
+    const int xfr = XR >= 16 ? fr : (fr < XR ? fr : XR - 1);   // ... the staged X row this lane reads
 
 #define OPMX_STEP(SET, KCI)                                                                            \
     do {                                                                                               \
@@ -169,7 +178,7 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
             _Pragma("unroll") for (int g = 0; g < NG; ++g)                                             \
                 a_[g] = *reinterpret_cast<const frag *>(wstrip + (g * 16 + fr) * RS + c_ * 16);        \
             _Pragma("unroll") for (int m = 0; m < MT; ++m) {                                           \
-                const frag b_ = *reinterpret_cast<const frag *>(xcur_ + (m * 16 + fr) * RS + c_ * 16); \
+                const frag b_ = *reinterpret_cast<const frag *>(xcur_ + (m * 16 + xfr) * RS + c_ * 16); \
                 _Pragma("unroll") for (int g = 0; g < NG; ++g)                                         \
                     acc[g][m] = Mfma<T>::m16(a_[g], b_, acc[g][m]);                                    \
             }                                                                                          \
@@ -230,19 +239,19 @@ __global__ __launch_bounds__(SW * 64) void gemm_stream_kernel(const T *__restric
     }
 }
 
-template <typename T, int MT, int KC, int DEPTH, bool NT, int SW, bool SG, bool PAIR = false, bool SGW = false>
+template <typename T, int MT, int KC, int DEPTH, bool NT, int SW, bool SG, bool PAIR = false, bool SGW = false, int XR = 16 * MT>
 int stream_launch_sw(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
                      int64_t N, void *Y, hipStream_t s, RowGather g)
 {
     constexpr int SROWS = SGW ? 16 * SW / 2 : (PAIR ? 32 : 16) * SW;
     constexpr int RS = KC * 2 + 16;
-    constexpr int smem = SW * ((SG || PAIR) ? 2 : 1) * 16 * RS + 2 * 16 * MT * RS;
+    constexpr int smem = SW * ((SG || PAIR) ? 2 : 1) * 16 * RS + 2 * XR * RS;
     static_assert(!SGW || (SW / 2) * MT * 1024 <= smem, "the pair exchange reuses the staging memory");
-    auto kern = gemm_stream_kernel<T, MT, KC, DEPTH, NT, SW, SG, PAIR, SGW>;
+    auto kern = gemm_stream_kernel<T, MT, KC, DEPTH, NT, SW, SG, PAIR, SGW, XR>;
     static std::atomic<uint64_t> attr_done{0};
     if (!ensure_dynamic_smem(reinterpret_cast<const void *>(kern), smem, attr_done)) return OPMX_ERR_LAUNCH;
     dim3 grid(static_cast<unsigned>(ceil_div((SG || SGW) ? N / 2 : N, SROWS)),
-              static_cast<unsigned>(max_mtiles(R, E, 16 * MT)));
+              static_cast<unsigned>(max_mtiles(R, E, XR)));
     kern<<<grid, SW * 64, smem, s>>>(static_cast<const T *>(X), off, static_cast<const T *>(W),
                                      static_cast<const T *>(B), E, R, K, N, static_cast<T *>(Y), g.index, g.x_rows);
     OPMX_LAUNCH_CHECK();
@@ -267,8 +276,6 @@ int stream_launch(const void *X, const int64_t *off, const void *W, const void *
 
 // Row-tile height MT*16 from the rows-per-expert bound m; K-chunk width per height
 // (narrower chunks for taller tiles keep the LDS footprint, hence occupancy, level).
-// 32-row tiles are the measured sweet spot even for a handful of rows; the 16-row
-// instance only serves single-token calls.
 template <typename T, int KC1, int KC2, int KC4, int KC8, int DEPTH, bool NT>
 int stream_pick_mt(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
                    int64_t N, int64_t m, void *Y, hipStream_t s, RowGather g)
@@ -279,9 +286,20 @@ int stream_pick_mt(const void *X, const int64_t *off, const void *W, const void 
     // layer at T = 32 0.255 -> 0.211 ms, at T = 1 0.189 -> 0.126 ms).
     constexpr int KC1S = KC1 > 128 ? 128 : KC1, KC2S = KC2 > 128 ? 128 : KC2, KC4S = KC4 > 64 ? 64 : KC4;
     const bool short_k = K < 16 * 256;
-    if (m <= 2)
+    // Up to 8 rows per expert (twice the mean, or the caller's bound): 16-row tiles.  The X chunk a block
+    // stages is then half as large, which shows where blocks are single waves (few weight rows: the
+    // Mixtral down projection at T = 8 ... 12, 131 -> 126 us); no difference at T = 16 or with 64 experts.
+    if (m <= 8) {
+        // at most two rows in all (one token, two experts): two-row X tiles, see the kernel's XR
+        if constexpr (KC1 == 256 && DEPTH == 2 && NT)
+            if (R <= 2 && !short_k) {
+                if (ceil_div(N, 64) * R < 512)
+                    return stream_launch_sw<T, 1, 256, 2, true, 1, false, false, false, 2>(X, off, W, B, E, R, K, N, Y, s, g);
+                return stream_launch_sw<T, 1, 256, 2, true, 4, false, false, false, 2>(X, off, W, B, E, R, K, N, Y, s, g);
+            }
         return short_k ? stream_launch<T, 1, KC1S, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s, g)
                        : stream_launch<T, 1, KC1, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s, g);
+    }
     if (m <= 32)
         return short_k ? stream_launch<T, 2, KC2S, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s, g)
                        : stream_launch<T, 2, KC2, DEPTH, NT>(X, off, W, B, E, R, K, N, Y, s, g);
@@ -300,8 +318,11 @@ int stream_swiglu_impl(const void *X, const int64_t *off, const void *W, const v
 {
     const int64_t m = rows_hint > 0 ? rows_hint : R;
     if (m <= 2) {    // short K: narrower chunks, as in stream_pick_mt
-        if (K >= 16 * 256 && ceil_div(N / 2, 64) * (R < E ? R : E) >= 256)
+        if (K >= 16 * 256 && ceil_div(N / 2, 64) * (R < E ? R : E) >= 256) {
+            if (R <= 2)   // two-row X tiles, see the kernel's XR
+                return stream_launch_sw<T, 1, 256, 2, true, 4, false, false, true, 2>(X, off, W, B, E, R, K, N, Y, s, g);
             return stream_launch_sw<T, 1, 256, 2, true, 4, false, false, true>(X, off, W, B, E, R, K, N, Y, s, g);
+        }
         return K < 16 * 256 ? stream_launch<T, 1, 128, 2, true, true>(X, off, W, B, E, R, K, N, Y, s, g)
                             : stream_launch<T, 1, 256, 2, true, true>(X, off, W, B, E, R, K, N, Y, s, g);
     }

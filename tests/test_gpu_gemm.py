@@ -189,6 +189,21 @@ def test_tail_tiles_split_over_k(dtype):
         run_case("row", [200, 60], 9216, 4096, dtype, False, {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": "0"})
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_stream_two_row_tiles(dtype):
+    """Calls with at most two rows in all and K >= 4096 stage two X rows per tile instead of sixteen:
+    one token with two experts, two rows of one expert, a single row; one-wave and four-wave blocks
+    (few and many weight rows), a ragged last K chunk, bias, and the SwiGLU form by wave pairs
+    (N/2 >= 8192 columns for two active experts)."""
+    env = {"OPMX_MOE_GEMM": "stream"}
+    for sizes in ([1, 0, 1, 0, 0, 0, 0, 0], [0, 0, 0, 2, 0, 0, 0, 0], [0, 1], [1]):
+        run_case("column", sizes, 4096, 192, dtype, True, env)              # one-wave blocks
+        run_case("row", sizes, 4096 + 72, 320, dtype, False, env)           # ragged last chunk
+        run_case("column", sizes, 4096, 33000, dtype, True, env)            # four-wave blocks, N not a multiple of 64
+        run_case("column", sizes, 4096, 2 * 8256, dtype, True, env, swiglu=True)
+    run_case("column", [1, 0, 1, 0], 8192, 2 * 192, dtype, False, env, swiglu=True)   # few columns: the narrow SwiGLU form
+
+
 @pytest.mark.parametrize("variant", ["0", "1", "2", "3", "4", "5"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_stream_kernel_variants(variant, dtype):
