@@ -95,9 +95,8 @@ def measured_traffic(workload, forms):
 
 # configurations of the benchmark set measured beside the default workload (child processes), each as
 # the operator-by-operator sequence and with the fused forms MoeFeedForward uses by default
-COMPANIONS = [(w, f) for w in ("decode-T1", "decode-T8", "decode-T32", "decode-T128", "decode-T512", "decode-T1024",
-                               "prefill-T2048", "prefill-T8192", "fine-T32", "fine-T4096", "8x22b-T16", "8x22b-T4096")
-              for f in ([], ["--fused"]) if not (w == "decode-T32" and not f)]
+COMPANION_WORKLOADS = ["decode-T1", "decode-T8", "decode-T32", "decode-T128", "decode-T512", "decode-T1024",
+                       "prefill-T2048", "prefill-T8192", "fine-T32", "fine-T4096", "8x22b-T16", "8x22b-T4096"]
 
 
 SHAPES = {
@@ -149,6 +148,11 @@ def main():
                     help="MFMA-bound workloads: skip timing the vendor dense GEMM of the same flop count")
     ap.add_argument("--no-companion", action="store_true",
                     help="with the default workload, do not also measure the MFMA-bound prefill workload")
+    ap.add_argument("--companion-set", default="", metavar="W1,W2",
+                    help="measure only these workloads beside the default one (default: the whole benchmark set)")
+    ap.add_argument("--companion-file", default=os.path.join(ROOT, "gpurun_out", "bench_companions.json"),
+                    help="where the companion workloads' full records are written (the final line holds three "
+                         "figures per workload)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
                     help="also run N plain device-to-device copies of the gate/up weight tensor (known size): "
                          "the reference reading for FETCH_SIZE / WRITE_SIZE counter runs")
@@ -184,22 +188,40 @@ def main():
             print("device ceiling probe failed: {}".format(exc), file=sys.stderr)
     # The default run also measures every other configuration of the benchmark set: child
     # processes of this program, run one after the other while this one leaves the GPU idle.
+    # The final JSON line carries three figures per configuration (ms per step, whole-layer
+    # fraction of peak, dominant-kernel fraction of peak; [six operators, fused forms]); the
+    # children's full records go to stderr, one line each, and to --companion-file.
     companion = None
     if args.workload == "decode-T32" and not args.no_companion:
         import subprocess
-        companion = {}
-        for name, extra in COMPANIONS:
-            cmd = [sys.executable, os.path.abspath(__file__), "--workload", name, "--steps", "40", "--warmup", "5",
-                   "--windows", "2", "--conditioning-ms", "200", "--no-cpu-baseline", "--no-device-ceilings",
-                   "--no-vendor-gemm", "--no-companion"] + extra
-            try:
-                line = subprocess.run(cmd, capture_output=True, text=True, timeout=300, check=True).stdout.strip().splitlines()[-1]
-                r = json.loads(line)
-                companion[name + (", fused forms" if extra else "")] = {
-                    key: r[key] for key in ("value", "unit", "ms_per_step", "steps", "windows", "config", "roofline",
-                                            "layer", "hip_graph_replay", "per_op_us")}
-            except Exception as exc:
-                print("companion workload {} failed: {}".format(name, exc), file=sys.stderr)
+        names = [w.strip() for w in args.companion_set.split(",") if w.strip()] if args.companion_set else COMPANION_WORKLOADS
+        companion, full = {}, {}
+        for name in names:
+            entry = {"bound": None, "ms": [None, None], "layer_frac": [None, None], "kernel_frac": [None, None]}
+            for slot, extra in enumerate(([], ["--fused"])):
+                if name == "decode-T32" and not extra:
+                    continue            # the headline itself, filled in below
+                cmd = [sys.executable, os.path.abspath(__file__), "--workload", name, "--steps", "40", "--warmup", "5",
+                       "--windows", "2", "--conditioning-ms", "200", "--no-cpu-baseline", "--no-device-ceilings",
+                       "--no-vendor-gemm", "--no-companion"] + extra
+                try:
+                    line = subprocess.run(cmd, capture_output=True, text=True, timeout=300, check=True).stdout.strip().splitlines()[-1]
+                    r = json.loads(line)
+                    full[name + (", fused forms" if extra else "")] = r
+                    print("companion {}{}: {}".format(name, " --fused" if extra else "", line), file=sys.stderr)
+                    entry["bound"] = r["layer"]["bound"]
+                    entry["ms"][slot] = r["ms_per_step"]
+                    entry["layer_frac"][slot] = r["layer"]["frac"]
+                    entry["kernel_frac"][slot] = r["roofline"]["frac"]
+                except Exception as exc:
+                    print("companion workload {} failed: {}".format(name, exc), file=sys.stderr)
+            companion[name] = entry
+        try:
+            os.makedirs(os.path.dirname(os.path.abspath(args.companion_file)), exist_ok=True)
+            with open(args.companion_file, "w") as f:
+                json.dump(full, f, indent=1)
+        except OSError as exc:
+            print("companion records not written to {}: {}".format(args.companion_file, exc), file=sys.stderr)
 
     import torch_function as OPMX
     from model_zoo.mixtral.modeling.dynamic_batching.Model import MoeFeedForward
@@ -485,7 +507,37 @@ def main():
             "as_written": {"value": round(Tc / (spent_w / runs_w), 2), "unit": "tokens/s",
                            "sample": "{} run(s), routing bookkeeping in interpreted per-element loops as in the "
                                      "reference, {:.1f} s".format(runs_w, spent_w)}}
-    print(json.dumps(result))
+    if companion and "decode-T32" in companion:     # the headline is the six-operator form of this workload
+        c = companion["decode-T32"]
+        c["bound"], c["ms"][0], c["layer_frac"][0], c["kernel_frac"][0] = lay["bound"], result["ms_per_step"], lay["frac"], roof["frac"]
+    if companion:
+        result["companion_legend"] = ("per workload: ms per step, whole-layer and dominant-kernel fraction of the "
+                                      "peak named by bound; each as [six operators, fused forms]; full records: "
+                                      + os.path.relpath(args.companion_file, ROOT))
+    print(final_line(result))
+
+
+# The benchmark driver keeps the last 8 KB of stdout: the one JSON line must fit with room to spare.
+MAX_LINE = 6000
+OPTIONAL_KEYS = ("device_ceilings", "per_op_us", "companion_legend", "conditioning", "windows", "hip_graph_replay",
+                 "companion")
+
+
+def final_line(result):
+    """The JSON line of a result; while it is longer than MAX_LINE characters the largest of the
+    context-only keys is dropped (the keys the contract names are never dropped)."""
+    result = dict(result)
+    line = json.dumps(result)
+    dropped = []
+    while len(line) > MAX_LINE:
+        sizes = sorted((len(json.dumps(result[key])), key) for key in OPTIONAL_KEYS if result.get(key) is not None)
+        if not sizes:
+            break
+        result[sizes[-1][1]] = None
+        dropped.append(sizes[-1][1])
+        result["dropped_for_length"] = dropped
+        line = json.dumps(result)
+    return line
 
 
 if __name__ == "__main__":

@@ -81,6 +81,8 @@ enum Option {
     kOptGnx,             // OPMX_MOE_GEMM_GNX: tile order 0 / 4 / 8 / 16
     kOptStreamK,         // OPMX_MOE_GEMM_STREAMK: 0 never split the tail tiles over K, 2 whenever possible
     kOptPersist,         // OPMX_MOE_GEMM_PERSIST: 0 never the persistent form, 1 whenever possible
+    kOptRouteIndexTokens,  // OPMX_MOE_ROUTE_INDEX_TOKENS: up to how many tokens (0 ... 64) the index form of router
+                           // gate + MoeSelect runs as one launch of one block
     kNumOptions
 };
 int option(Option o);

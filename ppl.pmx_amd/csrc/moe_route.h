@@ -56,45 +56,22 @@ __device__ __forceinline__ void route_token(const T *srow, int E, int k, int G, 
         // so "how many keys beat mine" is the key's position in the descending order:
         // E scalar broadcasts and compares, no k-round dependency chain.  The key of
         // rank j then moves to lane j through LDS-free cross-lane reads.
-        int rank[kMaxVpl];
-#pragma unroll
-        for (int v = 0; v < kMaxVpl; ++v) rank[v] = 0;
-        if (vpl == 1) {                      // E <= 64: one key per lane
-            for (int sl = 0; sl < E; ++sl) {
-                const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[0]), sl);
-                const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[0] >> 32), sl);
-                rank[0] += ((static_cast<uint64_t>(hi) << 32) | lo) > keys[0] ? 1 : 0;
-            }
-        } else {
-#pragma unroll
-            for (int sv = 0; sv < kMaxVpl; ++sv) {
-                if (sv < vpl) {
-                    for (int sl = 0; sl < kWave; ++sl) {
-                        if (sl + sv * kWave >= E) break;
-                        const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[sv]), sl);
-                        const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[sv] >> 32), sl);
-                        const uint64_t other = (static_cast<uint64_t>(hi) << 32) | lo;
-#pragma unroll
-                        for (int v = 0; v < kMaxVpl; ++v) rank[v] += other > keys[v] ? 1 : 0;
-                    }
-                }
-            }
+        int rank = 0;
+        for (int sl = 0; sl < E; ++sl) {
+            const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[0]), sl);
+            const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[0] >> 32), sl);
+            rank += ((static_cast<uint64_t>(hi) << 32) | lo) > keys[0] ? 1 : 0;
         }
         // lane j < k fetches the key whose rank is j: every lane publishes (rank -> key) by ballot
-#pragma unroll
-        for (int v = 0; v < kMaxVpl; ++v) {
-            if (v < vpl) {
-                for (int j = 0; j < k; ++j) {
-                    const uint64_t hit = __ballot(rank[v] == j && keys[v] != 0ull);
-                    if (hit) {
-                        const int src = __ffsll(static_cast<long long>(hit)) - 1;
-                        const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[v]), src);
-                        const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[v] >> 32), src);
-                        if (lig == j) {
-                            my_id = static_cast<int>(0xFFFFFFFFu - lo);
-                            my_v = key_value(hi);
-                        }
-                    }
+        for (int j = 0; j < k; ++j) {
+            const uint64_t hit = __ballot(rank == j && keys[0] != 0ull);
+            if (hit) {
+                const int src = __ffsll(static_cast<long long>(hit)) - 1;
+                const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[0]), src);
+                const uint32_t hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(keys[0] >> 32), src);
+                if (lig == j) {
+                    my_id = static_cast<int>(0xFFFFFFFFu - lo);
+                    my_v = key_value(hi);
                 }
             }
         }

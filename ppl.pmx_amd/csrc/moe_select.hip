@@ -335,6 +335,120 @@ __global__ __launch_bounds__(1024) void select_small_kernel(const T *__restrict_
     expand_row(X, Xp, static_cast<int64_t>(me), H, k, my_inv, vec);
 }
 
+// ---- index form, few tokens: router gate, top-k, softmax, offsets, inverse permutation and
+// row_token in ONE launch of ONE block.  Without row copies (the gate/up GEMM reads X through
+// row_token) nothing in MoeSelect needs more than one block, and the bookkeeping needs every
+// token's picks, so a single block of sixteen waves does it all:
+//   1. logits on the MFMA 16x16x32 units: the tokens form TT tiles of 16, the 16 / TT waves of a tile
+//      split K (wave kw takes k-steps kw, kw + 16/TT, ...; four steps of loads in flight) and hold
+//      all ET expert tiles; partial sums meet in LDS and are added in wave order, + bias, rounded
+//      once to T (Linear.py:32) -- written to `scores` and kept in LDS;
+//   2. top-k / softmax per token by lane groups on the rounded logits (moe_route.h), bit matrix;
+//   3. word prefixes, scan over experts -> expert_offset;
+//   4. rank of every (token, slot) -> invert_permutation, row_token.
+// One CU pulls X and Wg at roughly 100-150 GB/s, so the launch costs a few microseconds per 16
+// tokens: it replaces two or three dependent launches up to kIndexOneLaunchTokens tokens.
+constexpr int kIndexWaves = 16;
+constexpr int kIndexMaxTokens = 64;          // what the kernel can do (four token tiles)
+template <typename T, int TT, int ET>
+__global__ __launch_bounds__(kIndexWaves * 64) void route_index_kernel(const T *__restrict__ X, const T *__restrict__ Wg,
+                                                                       const T *__restrict__ Bg, int Ttok, int64_t H,
+                                                                       int E, int k, int G, T *__restrict__ scores_out,
+                                                                       T *__restrict__ weights, int64_t *__restrict__ inv,
+                                                                       int64_t *__restrict__ off,
+                                                                       int32_t *__restrict__ row_token,
+                                                                       int32_t *__restrict__ ids_out)
+{
+    using frag = typename Mfma<T>::frag;
+    constexpr int NWK = kIndexWaves / TT;                    // waves that split K for one token tile
+    constexpr int kE = 64;                                   // experts this kernel handles (one key per lane)
+    extern __shared__ __attribute__((aligned(16))) char dyn[];
+    float *part = reinterpret_cast<float *>(dyn);            // [kIndexWaves][ET][64][4]
+    __shared__ T s_scores[kIndexMaxTokens * kE];
+    __shared__ uint32_t bits[kE * kWords];
+    __shared__ int wordpre[kE * kWords];
+    __shared__ int count[kE + 1];
+    __shared__ int s_ids[kIndexMaxTokens * OPMX_MOE_MAX_EXPERTS_PER_TOKEN];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int fr = lane & 15, fg = lane >> 4;
+    {
+        const int tt = wave % TT, kw = wave / TT;
+        const int trow = tt * 16 + fr < Ttok ? tt * 16 + fr : Ttok - 1;      // padded token rows repeat the last one
+        const T *xp = X + static_cast<int64_t>(trow) * H + fg * 8;
+        const T *wp[ET];
+#pragma unroll
+        for (int e = 0; e < ET; ++e) {
+            const int erow = e * 16 + fr < E ? e * 16 + fr : E - 1;            // padded expert rows likewise
+            wp[e] = Wg + static_cast<int64_t>(erow) * H + fg * 8;
+        }
+        float4_t acc[ET];
+#pragma unroll
+        for (int e = 0; e < ET; ++e) acc[e] = float4_t{0.f, 0.f, 0.f, 0.f};
+        const int steps = static_cast<int>(H / 32);
+        int st = kw;
+        for (; st + 3 * NWK < steps; st += 4 * NWK) {
+            frag b[4], a[4][ET];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                b[u] = *reinterpret_cast<const frag *>(xp + (st + NWK * u) * 32);
+#pragma unroll
+                for (int e = 0; e < ET; ++e) a[u][e] = *reinterpret_cast<const frag *>(wp[e] + (st + NWK * u) * 32);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int e = 0; e < ET; ++e) acc[e] = Mfma<T>::m16(a[u][e], b[u], acc[e]);
+        }
+        for (; st < steps; st += NWK) {
+            const frag b = *reinterpret_cast<const frag *>(xp + st * 32);
+#pragma unroll
+            for (int e = 0; e < ET; ++e) acc[e] = Mfma<T>::m16(*reinterpret_cast<const frag *>(wp[e] + st * 32), b, acc[e]);
+        }
+        // acc[e][i]: expert e*16 + fg*4 + i, token tt*16 + fr
+#pragma unroll
+        for (int e = 0; e < ET; ++e) *reinterpret_cast<float4_t *>(part + ((wave * ET + e) * 64 + lane) * 4) = acc[e];
+    }
+    zero_bits(bits, E);
+    __syncthreads();
+    for (int q = threadIdx.x; q < Ttok * E; q += blockDim.x) {
+        const int t = q / E, e = q - t * E;
+        const int tt = t >> 4, idx = (((e >> 4) * 64) + (((e & 15) >> 2) * 16 + (t & 15))) * 4 + (e & 3);
+        float v = 0.0f;
+#pragma unroll
+        for (int kw = 0; kw < NWK; ++kw) v += part[(kw * TT + tt) * ET * 64 * 4 + idx];
+        if (Bg) v += to_f32(Bg[e]);
+        const T r = from_f32<T>(v);
+        s_scores[q] = r;
+        scores_out[q] = r;
+    }
+    __syncthreads();
+    const int lig = threadIdx.x % G, grp = threadIdx.x / G, ngrp = kIndexWaves * 64 / G;
+    for (int tl = grp; tl < Ttok; tl += ngrp) {                 // whole lane groups iterate together
+        int id;
+        float w;
+        route_token(s_scores + tl * E, E, k, G, 1, lig, id, w);
+        if (lig < k) {
+            atomicOr(&bits[id * kWords + (tl >> 5)], 1u << (tl & 31));
+            s_ids[tl * k + lig] = id;
+            weights[tl * k + lig] = from_f32<T>(w);
+            if (ids_out) ids_out[tl * k + lig] = id;
+        }
+    }
+    __syncthreads();
+    word_prefix(bits, wordpre, count, E);
+    __syncthreads();
+    if (threadIdx.x < kWave) scan_experts(count, E);            // exclusive scan over experts, in place
+    __syncthreads();
+    for (int e = threadIdx.x; e <= E; e += blockDim.x) off[e] = count[e];
+    for (int q = threadIdx.x; q < Ttok * k; q += blockDim.x) {
+        const int t = q / k, e = s_ids[q];
+        const int pos = count[e] + rank_in_chunk(bits, wordpre, e, t);
+        inv[q] = pos;
+        row_token[pos] = t;
+    }
+}
+
 // The buffer select_impl keeps the picked ids in: the caller's, or a part of the workspace.
 inline int32_t *picks_buffer(int64_t Ttok, int E, int32_t *ids, void *ws)
 {
@@ -424,6 +538,45 @@ int route_select_fused(const void *X_, const void *Wg_, const void *Bg_, int64_t
     return OPMX_OK;
 }
 
+// Up to how many tokens route_index_kernel stands for the router kernel and the select kernels
+// (measured against them on the Mixtral shape and with 64 experts).
+constexpr int kIndexOneLaunchTokens = 32;
+
+template <typename T, int TT>
+int route_index_launch(const T *X, const T *Wg, const T *Bg, int Ttok, int64_t H, int E, int k, T *scores, T *w,
+                       int64_t *inv, int64_t *off, int32_t *row_token, int32_t *ids, hipStream_t s)
+{
+    int G = 8;
+    while (G < E) G <<= 1;                       // E <= 64: one key per lane
+    const int ET = (E + 15) / 16;
+    static std::atomic<uint64_t> attr_done[3];
+#define OPMX_ROUTE_INDEX(ETV, SLOT)                                                                         \
+    do {                                                                                                    \
+        auto kern = route_index_kernel<T, TT, ETV>;                                                         \
+        constexpr int smem = kIndexWaves * ETV * 64 * 4 * static_cast<int>(sizeof(float));                  \
+        if (!ensure_dynamic_smem(reinterpret_cast<const void *>(kern), smem, attr_done[SLOT])) return OPMX_ERR_LAUNCH; \
+        kern<<<1, kIndexWaves * 64, smem, s>>>(X, Wg, Bg, Ttok, H, E, k, G, scores, w, inv, off, row_token, ids); \
+    } while (0)
+    if (ET == 1) OPMX_ROUTE_INDEX(1, 0);
+    else if (ET == 2) OPMX_ROUTE_INDEX(2, 1);
+    else OPMX_ROUTE_INDEX(4, 2);
+#undef OPMX_ROUTE_INDEX
+    OPMX_LAUNCH_CHECK();
+    return OPMX_OK;
+}
+
+template <typename T>
+int route_index(const void *X, const void *Wg, const void *Bg, int64_t Ttok, int64_t H, int E, int k, void *scores,
+                void *w, int64_t *inv, int64_t *off, int32_t *row_token, int32_t *ids, hipStream_t s)
+{
+    const T *x = static_cast<const T *>(X), *wg = static_cast<const T *>(Wg), *bg = static_cast<const T *>(Bg);
+    T *sc = static_cast<T *>(scores), *wt = static_cast<T *>(w);
+    const int t = static_cast<int>(Ttok);
+    if (t <= 16) return route_index_launch<T, 1>(x, wg, bg, t, H, E, k, sc, wt, inv, off, row_token, ids, s);
+    if (t <= 32) return route_index_launch<T, 2>(x, wg, bg, t, H, E, k, sc, wt, inv, off, row_token, ids, s);
+    return route_index_launch<T, 4>(x, wg, bg, t, H, E, k, sc, wt, inv, off, row_token, ids, s);
+}
+
 }  // namespace
 
 // Router gate and MoeSelect in one call.  One launch when the logits of all tokens fit one
@@ -435,6 +588,14 @@ int launch_moe_route_select(const void *X, const void *Wg, const void *Bg, int64
 {
     const bool lowp = dtype == OPMX_DTYPE_F16 || dtype == OPMX_DTYPE_BF16;
     static_assert(kFusedMaxTokens <= kFusedTokens, "one MFMA tile of tokens");
+    static_assert(kIndexOneLaunchTokens <= kIndexMaxTokens, "four token tiles");
+    // Index form (no row copies), few tokens, up to 64 experts: everything in one launch of one block.
+    const int one_launch = option(kOptRouteIndexTokens) >= 0 ? option(kOptRouteIndexTokens) : kIndexOneLaunchTokens;
+    if (lowp && Xp == nullptr && row_token != nullptr && T >= 1 && T <= one_launch && T <= kIndexMaxTokens && E <= 64 &&
+        H >= 32 && H % 32 == 0 && aligned16(X) && aligned16(Wg)) {
+        if (dtype == OPMX_DTYPE_F16) return route_index<f16>(X, Wg, Bg, T, H, E, k, scores, w, inv, off, row_token, ids, s);
+        return route_index<bf16>(X, Wg, Bg, T, H, E, k, scores, w, inv, off, row_token, ids, s);
+    }
     if (lowp && T >= 1 && T <= kFusedMaxTokens && E <= kFusedExperts && H >= 32 && H % 32 == 0 && aligned16(X) &&
         aligned16(Wg)) {
         if (dtype == OPMX_DTYPE_F16)

@@ -75,28 +75,34 @@ class MoeFeedForward(nn.Module):
                                num_experts=num_experts, num_experts_per_token=num_experts_per_token)
 
     def _forward_indexed(self, x):
-        """The block with MoeSelect as an index (``fuse_x_gather``): same operator order as ``forward``."""
+        """The block with MoeSelect as an index (``fuse_x_gather``): same operator order as ``forward``.
+        -> (output, router logits)"""
         k, E = self.num_experts_per_token, self.num_experts
         if self.fuse_router_select:
-            expert_weights, invert_permutation, expert_offset, row_token, _ = OPMX.moe_route_select_index(
+            expert_weights, invert_permutation, expert_offset, row_token, router_logits = OPMX.moe_route_select_index(
                 x, self.gate.weight, self.gate.bias, E, k)
         else:
-            expert_weights, invert_permutation, expert_offset, row_token = OPMX.moe_select_index(self.gate(x), E, k)
+            router_logits = self.gate(x)
+            expert_weights, invert_permutation, expert_offset, row_token = OPMX.moe_select_index(router_logits, E, k)
         col = lambda m, swiglu=False: OPMX.moe_column_parallel_linear_indexed(
-            x, row_token, expert_offset, m.weight, m.bias, E, m.in_features, m.out_features, swiglu=swiglu)
+            x, row_token, expert_offset, m.weight, m.bias, E, m.in_features, m.out_features, swiglu=swiglu,
+            num_experts_per_token=k)
         if self.fused_ffn_glu:
             x13 = col(self.wu, True) if self.fuse_swiglu_epilogue else OPMX.swiglu(col(self.wu))
         else:
             x13 = OPMX.silu(col(self.w1), col(self.w3))
         x_out = self.w2(x13, expert_offset)
-        return OPMX.moe_reduce(x_out, expert_weights, invert_permutation, k)
+        return OPMX.moe_reduce(x_out, expert_weights, invert_permutation, k), router_logits
 
-    def forward(self, x):
+    def forward(self, x, return_router_logits: bool = False):
+        """``return_router_logits`` (not in the reference's signature, ``Model.py:187``): also return the
+        router logits ``[*, E]`` the tokens were routed by, as the block's router call computed them."""
         k = self.num_experts_per_token
         if self.fuse_x_gather and not torch.onnx.is_in_onnx_export():
-            return self._forward_indexed(x)
+            out, router_logits = self._forward_indexed(x)
+            return (out, router_logits) if return_router_logits else out
         if self.fuse_router_select and not torch.onnx.is_in_onnx_export():
-            x_experts, expert_weights, invert_permutation, expert_offset, _ = OPMX.moe_route_select(
+            x_experts, expert_weights, invert_permutation, expert_offset, router_logits = OPMX.moe_route_select(
                 x, self.gate.weight, self.gate.bias, self.num_experts, k)
         else:
             router_logits = self.gate(x)
@@ -112,7 +118,8 @@ class MoeFeedForward(nn.Module):
         else:
             x13 = OPMX.silu(self.w1(x_experts, expert_offset), self.w3(x_experts, expert_offset))
         x_out = self.w2(x13, expert_offset)
-        return OPMX.moe_reduce(x_out, expert_weights, invert_permutation, k)
+        out = OPMX.moe_reduce(x_out, expert_weights, invert_permutation, k)
+        return (out, router_logits) if return_router_logits else out
 
     @torch.no_grad()
     def load_state_dict(self, state_dict, strict: bool = True, prefix=None):

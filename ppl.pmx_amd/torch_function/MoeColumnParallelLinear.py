@@ -52,12 +52,16 @@ def moe_column_parallel_linear_swiglu(X, expert_offset, W, B, num_experts: int, 
 
 
 def moe_column_parallel_linear_indexed(X, row_token, expert_offset, W, B, num_experts: int, in_features: int,
-                                       out_features: int, swiglu: bool = False) -> torch.Tensor:
+                                       out_features: int, swiglu: bool = False,
+                                       num_experts_per_token: int = 0) -> torch.Tensor:
     """``moe_column_parallel_linear`` (or its SwiGLU form) on the rows ``X[row_token]``: ``X`` ``[*, K]``
     holds the tokens, ``row_token`` is the int32 index ``moe_select_index`` returns in place of
     ``X_expand_permute``.  Bit for bit the result of the operator on ``X_expand_permute``
     (``MoeSelect.py:45-47`` followed by ``MoeColumnParallelLinear.py:58-67``), ``[*, k, N]``, without the
-    ``[T*k, K]`` copy ever being written or read.  No counterpart operator in the reference; eager only."""
+    ``[T*k, K]`` copy ever being written or read.  ``num_experts_per_token`` only shapes the (empty)
+    result of an empty batch, where ``row_token`` does not tell k.  No counterpart operator in the
+    reference; eager only."""
     assert X.shape[-1] == in_features, "X.shape is {}, in_features is {}".format(X.shape, in_features)
     return grouped_linear("column", X, expert_offset, W, B, num_experts,
-                          epilogue=_lib.EPILOGUE_SWIGLU if swiglu else _lib.EPILOGUE_NONE, row_index=row_token)
+                          epilogue=_lib.EPILOGUE_SWIGLU if swiglu else _lib.EPILOGUE_NONE, row_index=row_token,
+                          rows_per_token=num_experts_per_token)

@@ -4,7 +4,8 @@ import torch
 from . import _lib
 
 
-def grouped_linear(op, X, expert_offset, W, B, num_experts, epilogue=_lib.EPILOGUE_NONE, row_index=None):
+def grouped_linear(op, X, expert_offset, W, B, num_experts, epilogue=_lib.EPILOGUE_NONE, row_index=None,
+                   rows_per_token=0):
     """``Y[off[e]:off[e+1]] = X[off[e]:off[e+1]] @ W[e]^T (+ B[e])`` on the GPU.
 
     ``op`` is "column" or "row".  Output dtype is ``W.dtype`` on ``X.device``
@@ -14,7 +15,7 @@ def grouped_linear(op, X, expert_offset, W, B, num_experts, epilogue=_lib.EPILOG
     ``row_index`` (int32 ``[R]``, column form only): GEMM row r is ``X.view(-1, K)[row_index[r]]``
     -- X holds the tokens and ``row_index`` is the ``row_token`` output of ``moe_select_index``;
     the result then has the shape ``[*, R / tokens, N]`` that the operator gives on
-    ``X_expand_permute``.
+    ``X_expand_permute`` (an empty batch has no such ratio: ``rows_per_token`` names it then).
     """
     name = "moe_{}_parallel_linear".format(op)
     dev = _lib.require_gpu(name, X, expert_offset, W, B, row_index)
@@ -38,7 +39,7 @@ def grouped_linear(op, X, expert_offset, W, B, num_experts, epilogue=_lib.EPILOG
     if row_index is not None:
         if op != "column" or row_index.dtype != torch.int32 or row_index.dim() != 1:
             raise ValueError("{}: row_index must be a 1-D int32 tensor (column form only)".format(name))
-        if tokens == 0 or row_index.numel() % tokens:
+        if (tokens == 0 and row_index.numel() != 0) or (tokens != 0 and row_index.numel() % tokens):
             raise ValueError("{}: row_index has {} entries for {} rows of X".format(name, row_index.numel(), tokens))
         row_index = row_index.contiguous()
     R = tokens if row_index is None else row_index.numel()
@@ -70,7 +71,7 @@ def grouped_linear(op, X, expert_offset, W, B, num_experts, epilogue=_lib.EPILOG
                                             dt, hint, _lib.ptr(Y), _lib.ptr(ws), ws_bytes, _lib.stream_ptr(dev))
     _lib.check(rc, name)
     if row_index is not None:
-        return Y.view(*X.shape[:-1], R // tokens, n_out)
+        return Y.view(*X.shape[:-1], R // tokens if tokens else int(rows_per_token), n_out)
     return Y.view(*X.shape[:-1], n_out)
 
 

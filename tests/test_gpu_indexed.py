@@ -50,23 +50,75 @@ def test_select_index_matches_oracle_and_select(T, H, E, k, dtype, ties):
     assert torch.equal(w.view(torch.uint8), w2.view(torch.uint8)) and torch.equal(inv, inv2) and torch.equal(off, off2)
 
 
-@pytest.mark.parametrize("T,H,E,k,dtype", [(1, 4096, 8, 2, torch.float16), (8, 4096, 8, 2, torch.float16),
-                                            (8, 2048, 16, 4, torch.bfloat16), (32, 4096, 8, 2, torch.float16),
-                                            (600, 512, 16, 2, torch.float16), (5, 96, 8, 2, torch.float32)])
-def test_route_select_index_matches_route_select(T, H, E, k, dtype):
-    """Router gate in front: same logits and routing as moe_route_select, which is oracle-checked."""
+ROUTE_INDEX_CASES = [
+    # one launch of one block (fp16 / bf16, up to 32 tokens and 64 experts): one, two token tiles; 1, 2, 4 expert tiles
+    (1, 4096, 8, 2, torch.float16), (8, 4096, 8, 2, torch.float16), (16, 4096, 8, 2, torch.float16),
+    (17, 4096, 8, 2, torch.float16), (32, 4096, 8, 2, torch.float16), (8, 2048, 16, 4, torch.bfloat16),
+    (32, 2048, 64, 8, torch.bfloat16), (5, 2048, 64, 8, torch.bfloat16), (31, 96, 33, 5, torch.float16),
+    (32, 6144, 24, 24, torch.float16), (3, 32, 3, 1, torch.bfloat16), (20, 64, 64, 32, torch.float16),
+    # beyond: the router kernel and the select kernels one after the other
+    (33, 4096, 8, 2, torch.float16), (64, 2048, 64, 8, torch.bfloat16), (600, 512, 16, 2, torch.float16),
+    (5, 96, 8, 2, torch.float32), (16, 40, 8, 2, torch.float16), (12, 512, 100, 4, torch.bfloat16),
+]
+
+
+def check_route_select_index(T, H, E, k, dtype, bias=True, wscale=0.05, seed=None):
+    """moe_route_select_index against the oracle: logits within one rounding of the fp32 sum, and the
+    routing bit-exact on the logits the call itself returns."""
     OPMX = opmx()
-    g = torch.Generator().manual_seed(T + H)
-    X = torch.randn(T, H, generator=g).to(dtype).to(dev())
-    Wg = (torch.randn(E, H, generator=g) * 0.05).to(dtype).to(dev())
-    Bg = torch.randn(E, generator=g).to(dtype).to(dev())
+    g = torch.Generator().manual_seed(T + H if seed is None else seed)
+    Xc = torch.randn(T, H, generator=g).to(dtype)
+    Wgc = (torch.randn(E, H, generator=g) * wscale).to(dtype)
+    Bgc = torch.randn(E, generator=g).to(dtype) if bias else None
+    X, Wg, Bg = Xc.to(dev()), Wgc.to(dev()), None if Bgc is None else Bgc.to(dev())
     w, inv, off, row_token, scores = OPMX.moe_route_select_index(X, Wg, Bg, E, k)
-    xe2, w2, inv2, off2, scores2 = OPMX.moe_route_select(X, Wg, Bg, E, k)
-    assert torch.equal(scores, scores2) and torch.equal(inv, inv2) and torch.equal(off, off2)
-    assert torch.equal(w.view(torch.uint8), w2.view(torch.uint8))
-    assert torch.equal(X[row_token.long()], xe2.view(T * k, H))
-    rxe, rw, rinv, roff = O.moe_select(X.cpu(), scores.cpu(), E, k)
+    assert scores.shape == (T, E) and scores.dtype == dtype and row_token.dtype == torch.int32
+    ref = O.linear(Xc, Wgc, Bgc, out_dtype=torch.float32)
+    assert_close_ulp(scores, ref, dtype, ulps=2.0 if dtype != torch.float32 else 64.0, what="router logits")
+    rxe, rw, rinv, roff = O.moe_select(Xc, scores.cpu(), E, k)
     assert torch.equal(inv.cpu(), rinv) and torch.equal(off.cpu(), roff)
+    assert torch.equal(Xc[row_token.cpu().long()].view(torch.uint8), rxe.reshape(T * k, H).contiguous().view(torch.uint8))
+    assert float((w.cpu().double() - rw.double()).abs().max()) <= {torch.float32: 1e-6, torch.float16: 1e-3,
+                                                                   torch.bfloat16: 8e-3}[dtype]
+    # the same routing, bit for bit, as moe_select_index fed those logits
+    w2, inv2, off2, rt2 = OPMX.moe_select_index(scores, E, k)
+    assert torch.equal(w.view(torch.uint8), w2.view(torch.uint8)) and torch.equal(inv, inv2)
+    assert torch.equal(off, off2) and torch.equal(row_token, rt2)
+    return scores
+
+
+@pytest.mark.parametrize("T,H,E,k,dtype", ROUTE_INDEX_CASES)
+def test_route_select_index_matches_oracle(T, H, E, k, dtype):
+    check_route_select_index(T, H, E, k, dtype, bias=True)
+    check_route_select_index(T, H, E, k, dtype, bias=False, wscale=H ** -0.5, seed=7 * T + E)
+
+
+def test_route_select_index_one_launch_up_to_64_tokens():
+    """The one-launch kernel's four-token-tile form (33 ... 64 tokens), switched on through its knob."""
+    from torch_function import _lib
+    _lib.set_option("OPMX_MOE_ROUTE_INDEX_TOKENS", 64)
+    try:
+        for T, H, E, k, dtype in [(33, 4096, 8, 2, torch.float16), (64, 2048, 64, 8, torch.bfloat16),
+                                  (49, 512, 40, 6, torch.float16)]:
+            check_route_select_index(T, H, E, k, dtype)
+        _lib.set_option("OPMX_MOE_ROUTE_INDEX_TOKENS", 0)       # never: the separate kernels
+        check_route_select_index(8, 4096, 8, 2, torch.float16)
+    finally:
+        _lib.set_option("OPMX_MOE_ROUTE_INDEX_TOKENS", None)
+
+
+def test_route_select_index_ties_go_to_the_lower_expert():
+    """Identical gate rows give identical logits for every token: all picks are ties."""
+    T, H, E, k = 24, 64, 8, 3
+    g = torch.Generator().manual_seed(5)
+    X = torch.randn(T, H, generator=g).half()
+    Wg = torch.randn(1, H, generator=g).half().repeat(E, 1)
+    w, inv, off, row_token, scores = opmx().moe_route_select_index(X.to(dev()), Wg.to(dev()), None, E, k)
+    assert torch.equal(scores[:, :1].expand(T, E), scores)
+    assert off.cpu().tolist() == [0, T, 2 * T, 3 * T] + [3 * T] * (E - 3)
+    assert row_token.cpu().tolist() == list(range(T)) * 3
+    rxe, rw, rinv, roff = O.moe_select(X, scores.cpu(), E, k)
+    assert torch.equal(inv.cpu(), rinv)
 
 
 def offsets(sizes, lo=0):
@@ -167,6 +219,19 @@ def test_indexed_rejects_bad_arguments():
     assert bool(torch.isfinite(y.float()).all())
 
 
+def test_indexed_gemm_on_an_empty_batch():
+    import torch_function as OPMX
+    W = torch.zeros(4, 32, 64, dtype=torch.float16, device=dev())
+    X = torch.zeros(0, 64, dtype=torch.float16, device=dev())
+    rt = torch.zeros(0, dtype=torch.int32, device=dev())
+    off = torch.zeros(5, dtype=torch.int64, device=dev())
+    assert OPMX.moe_column_parallel_linear_indexed(X, rt, off, W, None, 4, 64, 32, num_experts_per_token=2).shape == (0, 2, 32)
+    assert OPMX.moe_column_parallel_linear_indexed(X, rt, off, W, None, 4, 64, 32, swiglu=True,
+                                                   num_experts_per_token=2).shape == (0, 2, 16)
+    with pytest.raises(ValueError):      # rows that name tokens of an empty X
+        OPMX.moe_column_parallel_linear_indexed(X, torch.zeros(2, dtype=torch.int32, device=dev()), off, W, None, 4, 64, 32)
+
+
 @pytest.mark.parametrize("T,H,E,k,I,dtype,skew", [
     (32, 4096, 8, 2, 14336, torch.float16, 0.0), (128, 4096, 8, 2, 14336, torch.float16, 0.0),
     (2048, 4096, 8, 2, 14336, torch.float16, 1.5), (4096, 2048, 64, 8, 1408, torch.bfloat16, 0.0),
@@ -174,7 +239,7 @@ def test_indexed_rejects_bad_arguments():
 def test_layer_with_the_gather_folded_into_the_gemm(T, H, E, k, I, dtype, skew):
     """Benchmark-shaped blocks: with the gather folded into the gate/up GEMM the block gives the bits
     of the operator-by-operator block, alone and together with the other fused forms (those
-    against the oracle, through the operator sequence's logits)."""
+    against the oracle, routed by the logits the block's own router call returned)."""
     from test_gpu_layer import build_layer, check_fused_against_oracle, run_ops
     (x, Wg, wu, w2), host = gpu_inputs(T, H, E, I, dtype, seed=7)
     bias = O.zipf_router_bias(E, skew).to(dtype) if skew else None
@@ -191,6 +256,4 @@ def test_layer_with_the_gather_folded_into_the_gemm(T, H, E, k, I, dtype, skew):
     for route in (False, True):
         mf = layer(fuse=True, route=route)
         mf.fuse_x_gather = True
-        if route and T <= 8:
-            continue         # one-launch router: routed by its own logits, covered in test_gpu_layer.py
-        check_fused_against_oracle(mf(x), g, host, E, k, full=T <= 2048)
+        check_fused_against_oracle(mf, x, host, E, k, bias=bias, full=T <= 2048)

@@ -5,6 +5,8 @@ workspace, so both are called through the C ABI on the same inputs and every out
 bit for bit (integers, weights and row copies alike: the kernels are the same).  Two calls in a
 row share the array, the second one smaller than the first, so stale contents of the first
 call sit behind the part the second one uses; the oracle checks the second call as well.
+Further down: the two calls enqueued back to back with no synchronisation between them, the
+allocator's byte count across a call, and the call captured into a HIP graph and replayed.
 """
 import pytest
 import torch
@@ -21,9 +23,7 @@ CALLS = [
 ]
 
 
-def _call(fn_name, X, s, E, k, with_ids):
-    from torch_function import _lib
-    L = _lib.lib()
+def _outputs(X, s, E, k, with_ids):
     T, H = X.shape
     d = X.device
     xe = torch.full((T * k, H), float("nan"), dtype=X.dtype, device=d)
@@ -31,18 +31,44 @@ def _call(fn_name, X, s, E, k, with_ids):
     inv = torch.full((T * k,), -7, dtype=torch.int64, device=d)
     off = torch.full((E + 1,), -7, dtype=torch.int64, device=d)
     ids = torch.full((T, k), -7, dtype=torch.int32, device=d) if with_ids else None
-    dt = _lib.dtype_id(X, fn_name)
-    stream = _lib.stream_ptr(d)
-    if fn_name == "opmx_moe_select":
-        ws = _lib.workspace(L.opmx_moe_select_workspace_bytes(T, E, k), d)
-        rc = L.opmx_moe_select(_lib.ptr(X), _lib.ptr(s), T, H, E, k, dt, _lib.ptr(xe), _lib.ptr(w), _lib.ptr(inv),
-                               _lib.ptr(off), _lib.ptr(ids), _lib.ptr(ws), ws.numel(), stream)
-    else:
-        rc = L.opmx_moe_select_static(_lib.ptr(X), _lib.ptr(s), T, H, E, k, dt, _lib.ptr(xe), _lib.ptr(w),
-                                      _lib.ptr(inv), _lib.ptr(off), _lib.ptr(ids), stream)
-    assert rc == 0, (fn_name, rc)
-    torch.cuda.synchronize()
     return xe, w, inv, off, ids
+
+
+def _enqueue_static(X, s, E, k, outs):
+    """opmx_moe_select_static on torch's current stream into preallocated outputs; no synchronisation."""
+    from torch_function import _lib
+    L = _lib.lib()
+    T, H = X.shape
+    xe, w, inv, off, ids = outs
+    rc = L.opmx_moe_select_static(_lib.ptr(X), _lib.ptr(s), T, H, E, k, _lib.dtype_id(X, "select_static"), _lib.ptr(xe),
+                                  _lib.ptr(w), _lib.ptr(inv), _lib.ptr(off), _lib.ptr(ids), _lib.stream_ptr(X.device))
+    assert rc == 0, rc
+
+
+def _call(fn_name, X, s, E, k, with_ids):
+    from torch_function import _lib
+    L = _lib.lib()
+    T, H = X.shape
+    outs = _outputs(X, s, E, k, with_ids)
+    if fn_name == "opmx_moe_select":
+        xe, w, inv, off, ids = outs
+        ws = _lib.workspace(L.opmx_moe_select_workspace_bytes(T, E, k), X.device)
+        rc = L.opmx_moe_select(_lib.ptr(X), _lib.ptr(s), T, H, E, k, _lib.dtype_id(X, fn_name), _lib.ptr(xe), _lib.ptr(w),
+                               _lib.ptr(inv), _lib.ptr(off), _lib.ptr(ids), _lib.ptr(ws), ws.numel(),
+                               _lib.stream_ptr(X.device))
+        assert rc == 0, (fn_name, rc)
+    else:
+        _enqueue_static(X, s, E, k, outs)
+    torch.cuda.synchronize()
+    return outs
+
+
+def _inputs(n):
+    T, H, E, k, dtype = CALLS[n]
+    g = torch.Generator().manual_seed(100 + n)
+    X = torch.randn(T, H, generator=g).to(dtype)
+    s = tie_heavy_scores(T, E, dtype, seed=n) if n == 0 else torch.randn(T, E, generator=g).to(dtype)
+    return X.to(dev()), s.to(dev()), E, k
 
 
 def _same_bits(a, b):
@@ -80,3 +106,44 @@ def test_static_scratch_select_few_tokens_and_empty():
         ref = _call("opmx_moe_select", X, s, E, k, False)
         for a, b in zip(got[:4], ref[:4]):
             assert _same_bits(a, b)
+
+
+def test_static_scratch_select_back_to_back_without_sync_and_without_allocation():
+    """The larger and the smaller call enqueued one behind the other on one stream with nothing
+    between them (the second overwrites the front of the scratch array as soon as the first is done
+    with it: stream order is the only protection, and it is enough), and the allocator's byte
+    count does not move across the two calls."""
+    a, b = _inputs(0), _inputs(1)
+    _call("opmx_moe_select_static", *a, True)               # first use on this GPU: symbol lookup, kernel attributes
+    outs_a, outs_b = _outputs(*a, True), _outputs(*b, True)
+    torch.cuda.synchronize()
+    before = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved())
+    _enqueue_static(*a, outs_a)
+    _enqueue_static(*b, outs_b)
+    after = (torch.cuda.memory_allocated(), torch.cuda.memory_reserved())
+    torch.cuda.synchronize()
+    assert before == after
+    for args, outs in ((a, outs_a), (b, outs_b)):
+        for got, ref in zip(outs, _call("opmx_moe_select", *args, True)):
+            assert _same_bits(got, ref)
+
+
+def test_static_scratch_select_captured_in_a_hip_graph():
+    """After one call outside capture (kernel attributes, the scratch address) the entry point only
+    enqueues kernels, so it records into a HIP graph; every replay, with eager calls of another size
+    and synchronisation in between, gives the eager bits."""
+    X, s, E, k = _inputs(0)
+    ref = _call("opmx_moe_select_static", X, s, E, k, True)
+    outs = _outputs(X, s, E, k, True)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _enqueue_static(X, s, E, k, outs)
+    for replay in range(3):
+        for t in outs:
+            t.fill_(-3)
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(outs, ref):
+            assert _same_bits(got, want), "replay {}".format(replay)
+        _call("opmx_moe_select_static", *_inputs(1), False)     # eager work on the same scratch array in between
