@@ -25,9 +25,12 @@ already resident in HBM.  Prints ONE JSON line:
                        MFMA-bound workloads: the vendor library's dense GEMM with the flop
                        count of the gate/up launch (no expert grouping), context only
   companion            with the default workload: every configuration of the benchmark set
-                       (decode T=1/8/32/128, T=512/1024, prefill T=2048/8192, 64 experts T=32/4096,
-                       8x22B shape T=16/4096), each as the operator-by-operator sequence and with the
-                       fused forms (--fused), measured by child processes of this program
+                       (fp32 T=64, decode T=1/8/32/128, T=512/1024, prefill T=2048/8192, 64 experts
+                       T=32/4096, 8x22B shape T=16/4096), each as the operator-by-operator sequence and
+                       with the fused forms (--fused), measured by child processes of this program: per
+                       workload ms per step, whole-layer and dominant-kernel fraction of peak, as
+                       [six operators, fused forms]; the children's full records go to stderr and to
+                       --companion-file
   cpu_baseline         the CPU oracle (PyTorch CPU restatement of the reference
                        operator sequence) on the host cores, bounded sample
 
@@ -38,7 +41,8 @@ drawn on the device unless --cpu-weights asks for the CPU draws as well (about a
 
 Workloads (--workload): decode-T{1,8,32,128} and prefill-T{2048,8192} at the
 Mixtral-8x7B shape (fp16), fine-T{32,4096} (64 experts, top-8, bf16),
-8x22b-T{16,4096}; e128-T<n> / e256-T<n>: 128 / 256 small experts (bf16).  Any T is accepted.
+8x22b-T{16,4096}; tiny-T64 (the fp32 configuration: hidden 1024, 8 experts, ffn 2816);
+e128-T<n> / e256-T<n>: 128 / 256 small experts (bf16).  Any T is accepted.
 Default: decode-T32, the configuration the metric is quoted on.
 """
 import argparse
@@ -54,6 +58,7 @@ for p in (ROOT, os.path.join(ROOT, "ppl.pmx_amd")):
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, vendor figure
 MFMA_PEAK_TFLOPS = 2500.0      # dense fp16/bf16 MFMA, vendor figure
+MFMA_PEAK_TFLOPS_F32 = 157.3   # dense fp32 MFMA, vendor figure
 
 # HBM bytes per launch of the dominant kernel come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # of this program, each scaled by the same counter's reading for a plain copy kernel of known size.
@@ -95,7 +100,7 @@ def measured_traffic(workload, forms):
 
 # configurations of the benchmark set measured beside the default workload (child processes), each as
 # the operator-by-operator sequence and with the fused forms MoeFeedForward uses by default
-COMPANION_WORKLOADS = ["decode-T1", "decode-T8", "decode-T32", "decode-T128", "decode-T512", "decode-T1024",
+COMPANION_WORKLOADS = ["tiny-T64", "decode-T1", "decode-T8", "decode-T32", "decode-T128", "decode-T512", "decode-T1024",
                        "prefill-T2048", "prefill-T8192", "fine-T32", "fine-T4096", "8x22b-T16", "8x22b-T4096"]
 
 
@@ -104,6 +109,8 @@ SHAPES = {
     "prefill": dict(H=4096, E=8, k=2, I=14336, dtype="float16", skew=1.5, name="mixtral-8x7b"),
     "fine": dict(H=2048, E=64, k=8, I=1408, dtype="bfloat16", skew=0.0, name="fine-grained-64x8"),
     "8x22b": dict(H=6144, E=8, k=2, I=16384, dtype="float16", skew=0.0, name="mixtral-8x22b-shape"),
+    # the reference's CPU-runnable configuration (fp32): parity case first, here also a measured one
+    "tiny": dict(H=1024, E=8, k=2, I=2816, dtype="float32", skew=0.0, name="tiny-fp32"),
     "decodebf": dict(H=4096, E=8, k=2, I=14336, dtype="bfloat16", skew=0.0, name="mixtral-8x7b-bf16"),
     "prefillbf": dict(H=4096, E=8, k=2, I=14336, dtype="bfloat16", skew=1.5, name="mixtral-8x7b-bf16"),
     # further shapes (not part of the reference's configurations): many small experts
@@ -229,7 +236,8 @@ def main():
     cfg = parse_workload(args.workload)
     T, H, E, k, I = cfg["T"], cfg["H"], cfg["E"], cfg["k"], cfg["I"]
     dtype = getattr(torch, cfg["dtype"])
-    s = 2
+    s = 4 if cfg["dtype"] == "float32" else 2
+    mfma_peak = MFMA_PEAK_TFLOPS_F32 if cfg["dtype"] == "float32" else MFMA_PEAK_TFLOPS
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
@@ -435,7 +443,7 @@ def main():
     fl = (args.fuse_swiglu, args.fuse_gather, args.fuse_router_select)
     forms = {(False, False, False): "none", (True, False, False): "swiglu", (True, True, True): "all"}.get(fl, "other")
     traffic, traffic_source = measured_traffic(args.workload, forms)
-    hbm_bound = (layer_flops / layer_bytes) < (MFMA_PEAK_TFLOPS * 1e12) / (HBM_PEAK_GBS * 1e9)
+    hbm_bound = (layer_flops / layer_bytes) < (mfma_peak * 1e12) / (HBM_PEAK_GBS * 1e9)
     if hbm_bound:
         ach = gemm1_bytes / (gemm1_ms * 1e-3) / 1e9
         roof = dict(bound="hbm", kernel="gate_up_grouped_gemm", achieved=round(ach, 1), peak=HBM_PEAK_GBS,
@@ -447,13 +455,13 @@ def main():
                    frac=round(lach / HBM_PEAK_GBS, 4), algorithmic_bytes=int(layer_bytes))
     else:
         ach = gemm1_flops / (gemm1_ms * 1e-3) / 1e12
-        roof = dict(bound="mfma", kernel="gate_up_grouped_gemm", achieved=round(ach, 1), peak=MFMA_PEAK_TFLOPS,
-                    unit="TFLOP/s", frac=round(ach / MFMA_PEAK_TFLOPS, 4),
+        roof = dict(bound="mfma", kernel="gate_up_grouped_gemm", achieved=round(ach, 1), peak=mfma_peak,
+                    unit="TFLOP/s", frac=round(ach / mfma_peak, 4),
                     traffic=traffic, traffic_source=traffic_source,
                     algorithmic_flops=int(gemm1_flops), launch_ms=round(gemm1_ms, 4))
         lach = layer_flops / (ms_per_step * 1e-3) / 1e12
-        lay = dict(bound="mfma", achieved=round(lach, 1), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
-                   frac=round(lach / MFMA_PEAK_TFLOPS, 4), algorithmic_flops=int(layer_flops))
+        lay = dict(bound="mfma", achieved=round(lach, 1), peak=mfma_peak, unit="TFLOP/s",
+                   frac=round(lach / mfma_peak, 4), algorithmic_flops=int(layer_flops))
 
     if ceilings:
         if hbm_bound:
@@ -468,7 +476,7 @@ def main():
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "conditioning": {"steps": cond_steps, "ms": round(cond_ms, 1), "timed": False}, "windows": windows,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": {"float16": "f16", "bfloat16": "bf16"}[cfg["dtype"]], "data": "synthetic",
+        "dtype": {"float16": "f16", "bfloat16": "bf16", "float32": "f32"}[cfg["dtype"]], "data": "synthetic",
         "config": {"workload": "{} MoE layer {}, T={} tokens, hidden={}, experts={}, top-{}, ffn={}, TP=1".format(
             cfg["name"], "decode" if hbm_bound else "prefill", T, H, E, k, I),
             "path": "drop-in operator sequence" + (" + fused SwiGLU epilogue" if args.fuse_swiglu else "")

@@ -129,6 +129,9 @@ int launch_grouped_gemm(const void *X, const int64_t *off, const void *W, const 
         return launch_gemm_tiled(X, off, W, B, E, R, K, N, dtype, epilogue,
                                  option(kOptTiledVariant) < 0 ? dflt : option(kOptTiledVariant), Y, ws, ws_bytes, s, g);
     }
+    // fp32 tensors: the fp32 matrix-unit kernel where its alignment conditions hold
+    if (dtype == OPMX_DTYPE_F32 && force != 1 && K > 0 && K % 4 == 0 && aligned16(X) && aligned16(W))
+        return launch_gemm_f32(X, off, W, B, E, R, K, N, epilogue, hint, Y, s, g);
     return launch_gemm_generic(X, off, W, B, E, R, K, N, dtype, epilogue, Y, s, g);
 }
 

@@ -187,6 +187,9 @@ __device__ __forceinline__ void zero_unowned_rows(T *__restrict__ Y, int64_t R, 
 
 int launch_gemm_generic(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R,
                         int64_t K, int64_t N, int dtype, int epilogue, void *Y, hipStream_t s, RowGather g = {});
+// fp32 tensors on the fp32 matrix units; requires K % 4 == 0 and 16-byte aligned X and W.
+int launch_gemm_f32(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
+                    int64_t N, int epilogue, int64_t rows_hint, void *Y, hipStream_t s, RowGather g = {});
 // variant: 0 = 256x256 direct-to-LDS kernel, 1 = 256x256 register-staged (8 waves),
 // 2 = 128x128 register-staged (4 waves).  off == nullptr: dense GEMM (one expert owns [0, R)).
 // ws / ws_bytes: optional scratch memory of gemm_tiled_workspace_bytes() bytes (variant 0 then

@@ -346,8 +346,14 @@ __global__ __launch_bounds__(1024) void select_small_kernel(const T *__restrict_
 //   2. top-k / softmax per token by lane groups on the rounded logits (moe_route.h), bit matrix;
 //   3. word prefixes, scan over experts -> expert_offset;
 //   4. rank of every (token, slot) -> invert_permutation, row_token.
-// One CU pulls X and Wg at roughly 100-150 GB/s, so the launch costs a few microseconds per 16
-// tokens: it replaces two or three dependent launches up to kIndexOneLaunchTokens tokens.
+// What bounds it is the one CU it runs on: a CU's load path moves 64 bytes per clock, so the logits
+// of 32 tokens (X 256 KB + Wg) cost it 8 us where the router kernel spreads them over 32 CUs.
+// Measured per call inside a HIP graph (router gate + MoeSelect, index form; separate kernels ->
+// this kernel): 8 experts, H = 4096: T = 1 7.3 -> 7.1 us, T = 8 8.7 -> 8.4, T = 16 8.2 -> 9.6, T = 32
+// 8.6 -> 15.5; 64 experts, H = 2048: T = 1 10.6 -> 13.8, T = 32 13.0 -> 32.6.  A dependent launch
+// costs about 4 us there, less than one CU needs for the logits of a second tile of tokens, so the
+// kernel is used up to kIndexOneLaunchTokens tokens and kIndexOneLaunchExperts experts and the
+// separate kernels (each on as many CUs as it has tokens) beyond.
 constexpr int kIndexWaves = 16;
 constexpr int kIndexMaxTokens = 64;          // what the kernel can do (four token tiles)
 template <typename T, int TT, int ET>
@@ -387,24 +393,23 @@ __global__ __launch_bounds__(kIndexWaves * 64) void route_index_kernel(const T *
         for (int e = 0; e < ET; ++e) acc[e] = float4_t{0.f, 0.f, 0.f, 0.f};
         const int steps = static_cast<int>(H / 32);
         int st = kw;
-        for (; st + 3 * NWK < steps; st += 4 * NWK) {
-            frag b[4], a[4][ET];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                b[u] = *reinterpret_cast<const frag *>(xp + (st + NWK * u) * 32);
-#pragma unroll
-                for (int e = 0; e < ET; ++e) a[u][e] = *reinterpret_cast<const frag *>(wp[e] + (st + NWK * u) * 32);
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
-#pragma unroll
-                for (int e = 0; e < ET; ++e) acc[e] = Mfma<T>::m16(a[u][e], b[u], acc[e]);
+        // U k-steps of loads in flight at a time: the phase costs about one memory round trip per batch
+#define OPMX_KBATCH(U)                                                                                     \
+        for (; st + ((U)-1) * NWK < steps; st += (U)*NWK) {                                                \
+            frag b[U], a[U][ET];                                                                           \
+            _Pragma("unroll") for (int u = 0; u < (U); ++u) {                                              \
+                b[u] = *reinterpret_cast<const frag *>(xp + (st + NWK * u) * 32);                          \
+                _Pragma("unroll") for (int e = 0; e < ET; ++e)                                             \
+                    a[u][e] = *reinterpret_cast<const frag *>(wp[e] + (st + NWK * u) * 32);                \
+            }                                                                                              \
+            _Pragma("unroll") for (int u = 0; u < (U); ++u)                                                \
+                _Pragma("unroll") for (int e = 0; e < ET; ++e) acc[e] = Mfma<T>::m16(a[u][e], b[u], acc[e]); \
         }
-        for (; st < steps; st += NWK) {
-            const frag b = *reinterpret_cast<const frag *>(xp + st * 32);
-#pragma unroll
-            for (int e = 0; e < ET; ++e) acc[e] = Mfma<T>::m16(*reinterpret_cast<const frag *>(wp[e] + st * 32), b, acc[e]);
-        }
+        if constexpr (ET == 1) OPMX_KBATCH(8)
+        OPMX_KBATCH(4)
+        OPMX_KBATCH(2)
+        OPMX_KBATCH(1)
+#undef OPMX_KBATCH
         // acc[e][i]: expert e*16 + fg*4 + i, token tt*16 + fr
 #pragma unroll
         for (int e = 0; e < ET; ++e) *reinterpret_cast<float4_t *>(part + ((wave * ET + e) * 64 + lane) * 4) = acc[e];
@@ -538,9 +543,9 @@ int route_select_fused(const void *X_, const void *Wg_, const void *Bg_, int64_t
     return OPMX_OK;
 }
 
-// Up to how many tokens route_index_kernel stands for the router kernel and the select kernels
-// (measured against them on the Mixtral shape and with 64 experts).
-constexpr int kIndexOneLaunchTokens = 32;
+// Up to how many tokens and experts route_index_kernel stands for the router kernel and the select
+// kernels (measured against them on the Mixtral shape and with 64 experts, see the kernel).
+constexpr int kIndexOneLaunchTokens = 8, kIndexOneLaunchExperts = 16;
 
 template <typename T, int TT>
 int route_index_launch(const T *X, const T *Wg, const T *Bg, int Ttok, int64_t H, int E, int k, T *scores, T *w,
@@ -590,8 +595,11 @@ int launch_moe_route_select(const void *X, const void *Wg, const void *Bg, int64
     static_assert(kFusedMaxTokens <= kFusedTokens, "one MFMA tile of tokens");
     static_assert(kIndexOneLaunchTokens <= kIndexMaxTokens, "four token tiles");
     // Index form (no row copies), few tokens, up to 64 experts: everything in one launch of one block.
-    const int one_launch = option(kOptRouteIndexTokens) >= 0 ? option(kOptRouteIndexTokens) : kIndexOneLaunchTokens;
-    if (lowp && Xp == nullptr && row_token != nullptr && T >= 1 && T <= one_launch && T <= kIndexMaxTokens && E <= 64 &&
+    // (the knob lifts both limits: up to 64 tokens and 64 experts, what the kernel can do)
+    const bool knob = option(kOptRouteIndexTokens) >= 0;
+    const int one_launch = knob ? option(kOptRouteIndexTokens) : kIndexOneLaunchTokens;
+    if (lowp && Xp == nullptr && row_token != nullptr && T >= 1 && T <= one_launch && T <= kIndexMaxTokens &&
+        E <= (knob ? 64 : kIndexOneLaunchExperts) &&
         H >= 32 && H % 32 == 0 && aligned16(X) && aligned16(Wg)) {
         if (dtype == OPMX_DTYPE_F16) return route_index<f16>(X, Wg, Bg, T, H, E, k, scores, w, inv, off, row_token, ids, s);
         return route_index<bf16>(X, Wg, Bg, T, H, E, k, scores, w, inv, off, row_token, ids, s);

@@ -51,7 +51,8 @@ def test_select_index_matches_oracle_and_select(T, H, E, k, dtype, ties):
 
 
 ROUTE_INDEX_CASES = [
-    # one launch of one block (fp16 / bf16, up to 32 tokens and 64 experts): one, two token tiles; 1, 2, 4 expert tiles
+    # one launch of one block (fp16 / bf16; by default up to 8 tokens and 16 experts, with the knob up to 64 and
+    # 64): one, two token tiles; 1, 2, 4 expert tiles
     (1, 4096, 8, 2, torch.float16), (8, 4096, 8, 2, torch.float16), (16, 4096, 8, 2, torch.float16),
     (17, 4096, 8, 2, torch.float16), (32, 4096, 8, 2, torch.float16), (8, 2048, 16, 4, torch.bfloat16),
     (32, 2048, 64, 8, torch.bfloat16), (5, 2048, 64, 8, torch.bfloat16), (31, 96, 33, 5, torch.float16),
@@ -88,9 +89,15 @@ def check_route_select_index(T, H, E, k, dtype, bias=True, wscale=0.05, seed=Non
 
 
 @pytest.mark.parametrize("T,H,E,k,dtype", ROUTE_INDEX_CASES)
-def test_route_select_index_matches_oracle(T, H, E, k, dtype):
-    check_route_select_index(T, H, E, k, dtype, bias=True)
-    check_route_select_index(T, H, E, k, dtype, bias=False, wscale=H ** -0.5, seed=7 * T + E)
+@pytest.mark.parametrize("one_launch_up_to", [None, 64])
+def test_route_select_index_matches_oracle(T, H, E, k, dtype, one_launch_up_to):
+    from torch_function import _lib
+    _lib.set_option("OPMX_MOE_ROUTE_INDEX_TOKENS", one_launch_up_to)
+    try:
+        check_route_select_index(T, H, E, k, dtype, bias=True)
+        check_route_select_index(T, H, E, k, dtype, bias=False, wscale=H ** -0.5, seed=7 * T + E)
+    finally:
+        _lib.set_option("OPMX_MOE_ROUTE_INDEX_TOKENS", None)
 
 
 def test_route_select_index_one_launch_up_to_64_tokens():
@@ -173,6 +180,12 @@ def test_indexed_generic_kernel(dtype, swiglu):
     env = {"OPMX_MOE_GEMM": "generic"}
     indexed_case(RAGGED8, 64, 72, 96, dtype, True, env, swiglu=swiglu)
     indexed_case([3, 200, 0, 7], 105, 50, 34, dtype, False, env, swiglu=swiglu)     # odd K and N; R = 2 T
+
+
+@pytest.mark.parametrize("swiglu", [False, True])
+def test_indexed_fp32_matrix_unit_kernel(swiglu):
+    indexed_case(RAGGED8, 64, 128, 96, torch.float32, True, swiglu=swiglu)         # 32-row tiles
+    indexed_case(BIG8, 2560, 100, 256, torch.float32, False, swiglu=swiglu)        # 128-row tiles, ragged K tile
 
 
 @pytest.mark.parametrize("variant", ["0", "1", "2", "3"])
