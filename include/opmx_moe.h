@@ -72,7 +72,7 @@ typedef enum opmx_epilogue {
 int opmx_moe_abi_version(void);
 const char *opmx_status_string(int status);
 
-/* Tuning / test knobs of the grouped GEMMs (no counterpart in the reference).  They choose
+/* Tuning / test knobs of the grouped GEMMs and the routing (no counterpart in the reference).  They choose
  * between kernels that compute the same thing; results change at most in accumulation order.
  * `name` is one of the strings below, `value` < 0 restores the automatic choice.  Each knob
  * starts from the environment variable of the same name, read once when the library is first
@@ -84,6 +84,8 @@ const char *opmx_status_string(int status);
  *   "OPMX_MOE_GEMM_GNX"            tile order: 8 expert-major, 16 row partition, 32 expert-grouped, 4, 0 row-major
  *   "OPMX_MOE_GEMM_STREAMK"        0 never split the tail tiles over K, 2 whenever possible
  *   "OPMX_MOE_GEMM_PERSIST"        0 never the persistent form, 1 whenever its conditions hold
+ *   "OPMX_MOE_ROUTE_INDEX_TOKENS"  up to how many tokens (0 ... 64, then also up to 64 experts)
+ *                                  opmx_moe_route_select_index runs as one launch of one block
  * Returns OPMX_ERR_BAD_ARGUMENT for an unknown name. */
 int opmx_moe_set_option(const char *name, int value);
 
@@ -136,11 +138,22 @@ int opmx_moe_select_static(const void *X, const void *scores, int64_t T, int64_t
  *   X [T,H], gate_weight [E,H], gate_bias [E] or NULL          (dtype)
  *   scores [T,E]: receives the router logits (an input of opmx_moe_select, an output here)
  *   the other outputs, the limits and the workspace are those of opmx_moe_select.
- * fp16/bf16 with T <= 8, E <= 16, H % 32 == 0 and 16-byte aligned X / gate_weight run as a
- * single launch (every block recomputes the few logits on the MFMA units); anything else runs
- * opmx_linear and opmx_moe_select one after the other.  Routing is exact on the returned
- * scores; the scores themselves may differ from opmx_linear's in the last bit (other
- * summation order of the fp32 accumulation). */
+ * Three regimes (fp16/bf16 with H % 32 == 0 and 16-byte aligned X / gate_weight; anything else, and
+ * float32, runs opmx_linear and opmx_moe_select one after the other):
+ *   T <= 8 and E <= 16   one launch: every block recomputes the few logits on the MFMA units, routes
+ *                        all tokens and emits its own token's outputs (the index form,
+ *                        opmx_moe_route_select_index, has no row copies to spread over blocks and
+ *                        runs as one block that does everything);
+ *   T > 256 and E <= 64  where the K-split MFMA router kernel serves the shape (see opmx_linear), it
+ *                        routes its 16 tokens per block in its epilogue -- top-k and softmax on the
+ *                        rounded logits it has just written -- and MoeSelect starts from the picks
+ *                        (histogram, scan, rank, row copies): one launch and the read-back of the
+ *                        logits less;
+ *   otherwise            the router kernel, then the MoeSelect kernels (a dependent launch costs
+ *                        about 4 us on this device; one block computing the logits of more than a
+ *                        handful of tokens costs more: a CU's load path moves 64 bytes per clock).
+ * Routing is exact on the returned scores in every regime; the scores themselves may differ from
+ * opmx_linear's in the last bit (other summation order of the fp32 accumulation). */
 int opmx_moe_route_select(const void *X, const void *gate_weight, const void *gate_bias, int64_t T,
                           int64_t H, int E, int k, int dtype, void *scores, void *X_expand_permute,
                           void *expert_weights, int64_t *invert_permutation, int64_t *expert_offset,
@@ -171,6 +184,9 @@ int opmx_moe_route_select_index(const void *X, const void *gate_weight, const vo
  * rows outside [off[0], off[E]) are set to zero.  expert_offset is read on the
  * device; it must be non-decreasing with values in [0, R].
  *   X [R,K], W [E,N,K], B [E,N] or NULL, Y [R,N] (or [R,N/2] with the SwiGLU epilogue).
+ * float16 / bfloat16 run on the fp16 / bf16 matrix units (weight-streaming kernel for few rows
+ * per expert, tile kernels beyond), float32 on the fp32 matrix units (K % 4 == 0, 16-byte aligned
+ * X and W); every other shape takes a shape-agnostic kernel.  Accumulation is fp32 throughout.
  * `rows_per_expert_hint` is the largest segment the caller can guarantee
  * (for MoeSelect output: min(R, T)); 0 = unknown.  It only selects between
  * kernel variants, never correctness.

@@ -902,6 +902,20 @@ __device__ __forceinline__ float4_t coherent_load(__amdgpu_buffer_rsrc_t slot, i
     return v;
 }
 
+// Scratch memory of the tail launch: arrival counters, then one fp32 tile-sized slot per workgroup.
+constexpr int kSkCounters = 256;                  // tail tiles are fewer than the CUs
+constexpr int kSkTile = 256 * 256;                // elements of an output tile
+
+// The arrival counters of the tail tiles must read zero when the tail launch starts.  The first
+// workgroup of the main launch clears them (count == nullptr: no tail launch follows): the tail
+// launch is ordered behind the main one on the stream, and a kernel's writes are visible to the
+// next kernel.  No memset and no launch of its own: callers may capture the sequence in a graph.
+__device__ __forceinline__ void clear_tail_counters(int *__restrict__ count)
+{
+    if (count != nullptr && blockIdx.x == 0)
+        for (int i = threadIdx.x; i < kSkCounters; i += blockDim.x) count[i] = 0;
+}
+
 // SK = false: one tile per workgroup (all tiles, or all but the tail when sk_wgs > 0 and the
 // tail is split).  SK = true: the tail launch, one k-range of one tail tile per workgroup.
 template <typename T, int BM, int BN, bool SWIGLU, bool SK>
@@ -931,6 +945,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
     __shared__ int s_arrivals;
     const int64_t ncols = SWIGLU ? N / 2 : N;
     if (!SK) zero_unowned_rows(Y, R, ncols, off, E);
+    if (!SK) clear_tail_counters(sk_count);
     stage_offsets(off, E, R, BM, s_off);
     const int mtiles = count_mtiles(off != nullptr, s_off, E, R, BM);
     const int nk = static_cast<int>(K / BK);
@@ -1256,6 +1271,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
                                                                        const T *__restrict__ Bias, int E, int64_t R,
                                                                        int64_t K, int64_t N, T *__restrict__ Y,
                                                                        int ntiles_n, int gnx, int sk_wgs, int sk_cost,
+                                                                       int *__restrict__ sk_count,
                                                                        const int32_t *__restrict__ rt, int64_t xrows)
 {
     constexpr int WM = 2, WN = 2, NW = 4;
@@ -1277,6 +1293,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
 
     const int64_t ncols = SWIGLU ? N / 2 : N;
     zero_unowned_rows(Y, R, ncols, off, E);
+    clear_tail_counters(sk_count);
     stage_offsets(off, E, R, BM, s_off);
     const int mtiles = count_mtiles(off != nullptr, s_off, E, R, BM);
     const int nk = static_cast<int>(K / BK);
@@ -1403,13 +1420,6 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
 #undef OPMX_XFRAG
 #undef OPMX_ISSUE1
 
-// Clears the arrival counters of the tail tiles (a kernel, not a memset: callers may capture
-// the launch sequence in a graph).
-__global__ void sk_clear_kernel(int *__restrict__ count, int n)
-{
-    for (int i = threadIdx.x; i < n; i += blockDim.x) count[i] = 0;
-}
-
 template <typename T, int BM, int BN, int WM, int WN>
 int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B, int E, int64_t R, int64_t K,
                    int64_t N, int epilogue, void *Y, hipStream_t s, RowGather g)
@@ -1440,10 +1450,6 @@ int tiled_launch(const void *X, const int64_t *off, const void *W, const void *B
     OPMX_LAUNCH_CHECK();
     return OPMX_OK;
 }
-
-// Scratch memory of the tail launch of the direct-to-LDS kernel.
-constexpr int kSkCounters = 256;                  // tail tiles are fewer than the CUs
-constexpr int kSkTile = 256 * 256;                // elements of an output tile
 
 // arrival counters, then one fp32 tile-sized slot per workgroup of the tail launch
 size_t sk_workspace_bytes(int cus)
@@ -1484,7 +1490,7 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
     if (option(kOptStreamK) == 0) sk_wgs = 0;    // tuning knob: 0 = off, 2 = split whenever possible
     if (option(kOptStreamK) == 2) sk_cost = 0;
     if (7 * (K / BK) <= 8 * sk_cost) sk_wgs = 0;     // sk_split() cannot split a K this short (g <= 8)
-    int *sk_count = static_cast<int *>(ws);
+    int *sk_count = sk_wgs > 0 ? static_cast<int *>(ws) : nullptr;      // nullptr: no tail launch, nothing to clear
     float *sk_part = reinterpret_cast<float *>(static_cast<char *>(ws) + kSkCounters * sizeof(int));
     dim3 grid(static_cast<unsigned>(dp_ids));
     dim3 block(256);
@@ -1516,7 +1522,7 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
         static std::atomic<uint64_t> attr_p[4];
         const bool hb = B != nullptr;
         using kernel_t = void (*)(const T *, const int64_t *, const T *, const T *, int, int64_t, int64_t, int64_t, T *, int,
-                                  int, int, int, const int32_t *, int64_t);
+                                  int, int, int, int *, const int32_t *, int64_t);
         const kernel_t kp = sw ? (hb ? gemm_tiled_dlds_persist_kernel<T, BM, BN, true, true>
                                      : gemm_tiled_dlds_persist_kernel<T, BM, BN, true, false>)
                                : (hb ? gemm_tiled_dlds_persist_kernel<T, BM, BN, false, true>
@@ -1525,8 +1531,7 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
         if (!ensure_dynamic_smem(reinterpret_cast<const void *>(kp), smem_p, attr_p[slot])) return OPMX_ERR_LAUNCH;
         // ids congruent mod 8 stay on one XCD as long as the grid is a multiple of 8
         const unsigned wgs = static_cast<unsigned>(dp_ids < cus ? dp_ids : cus);
-        if (sk_wgs > 0) sk_clear_kernel<<<1, 256, 0, s>>>(sk_count, kSkCounters);
-        kp<<<wgs, block, smem_p, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n, gnx, sk_wgs, sk_cost, g.index, g.x_rows);
+        kp<<<wgs, block, smem_p, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n, gnx, sk_wgs, sk_cost, sk_count, g.index, g.x_rows);
         if (sk_wgs > 0) {
             if (sw)
                 gemm_tiled_dlds_kernel<T, BM, BN, true, true><<<sk_wgs, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
@@ -1538,7 +1543,6 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
         OPMX_LAUNCH_CHECK();
         return OPMX_OK;
     }
-    if (sk_wgs > 0) sk_clear_kernel<<<1, 256, 0, s>>>(sk_count, kSkCounters);
     if (sw) {
         gemm_tiled_dlds_kernel<T, BM, BN, true, false><<<grid, block, smem, s>>>(Xp, off, Wp, Bp, E, R, K, N, Yp, ntiles_n,
                                                                                  gnx, sk_wgs, sk_cost, sk_part, sk_count, g.index, g.x_rows);

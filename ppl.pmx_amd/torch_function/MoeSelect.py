@@ -63,10 +63,12 @@ def moe_route_select(X: torch.Tensor, gate_weight: torch.Tensor, gate_bias, num_
     """Router gate and ``moe_select`` in one call (``Model.py:188-190`` of the reference:
     ``router_logits = self.gate(x)`` followed by ``OPMX.moe_select``).
 
-    -> the four outputs of ``moe_select`` plus the router logits ``[*, E]``.  Few tokens
-    (fp16/bf16, at most 8 tokens and 16 experts) run as a single launch; other sizes run the two
-    operators one after the other inside the library.  Not an ONNX node: a model that is being
-    exported calls ``linear`` and ``moe_select``.
+    -> the four outputs of ``moe_select`` plus the router logits ``[*, E]``.  Three regimes inside the
+    library (fp16/bf16): at most 8 tokens and 16 experts run as a single launch; beyond 256 tokens
+    (up to 64 experts) the router kernel routes its tokens in its epilogue and MoeSelect starts from
+    the picks; everything else runs the router kernel and the MoeSelect kernels one after the
+    other.  The routing is exact on the logits the call returns in every regime.  Not an ONNX node:
+    a model that is being exported calls ``linear`` and ``moe_select``.
     """
     E, k = int(num_experts), int(num_experts_per_token)
     lead, H = tuple(X.shape[:-1]), X.shape[-1]

@@ -6,7 +6,7 @@ operator allocates, synchronises or reads device data on the host, and if nothin
 records into the graph misbehaves on replay: every replay is checked bit for bit against an eager
 run on the same input, with eager work and synchronisation between the replays.  Cases cover the
 weight-streaming kernels, the tiled kernels with the split-K exchange (its counters are cleared by
-a kernel inside the graph), the persistent tiled kernel, and both select paths."""
+the main GEMM launch, inside the graph), the persistent tiled kernel, and both select paths."""
 import pytest
 import torch
 
