@@ -116,7 +116,7 @@ def check(path):
         if any(x.startswith("scratch_") for x in kloop):
             findings.append((name, "scratch access inside the k loop"))
         # 4. persistent kernel: the wait counts assume a fixed number of output stores per wave and
-        #    tile (16 or 32), the same number of priming stores before the tile loop, and no other
+        #    tile (8, 16 or 32), the same number of priming stores before the tile loop, and no other
         #    store in the loop
         if "persist" in name:
             thead = parent.get(khead)
@@ -132,7 +132,7 @@ def check(path):
                 tile = [l for l, h in zip(text, where) if inside(h)]
                 rest = [l for l, h in zip(text, where) if not inside(h)]
                 st = lambda part: sum(x.startswith("buffer_store_dwordx4") for x in part)
-                if st(rest) not in (16, 32) or st(tile) != st(rest):
+                if st(rest) not in (8, 16, 32) or st(tile) != st(rest):
                     findings.append((name, "{} priming stores, {} stores in the tile loop".format(st(rest), st(tile))))
                 # ... and that nothing in the tile loop drains the loads and stores kept in flight
                 # across tiles: no scratch traffic, no wait for all vector-memory operations

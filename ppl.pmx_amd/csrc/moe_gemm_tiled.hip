@@ -725,10 +725,12 @@ __device__ __forceinline__ constexpr int g2_load(bool wide, int m)              
 // in issue order, loads and stores alike).
 template <int N> __device__ __forceinline__ void wait_vm()
 {
-    static_assert(N == 0 || N == 12 || N == 16 || N == 32 || N == 48, "add the immediate here");
+    static_assert(N == 0 || N == 12 || N == 16 || N == 20 || N == 28 || N == 32 || N == 48, "add the immediate here");
     if (N == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     if (N == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
     if (N == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    if (N == 20) asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
+    if (N == 28) asm volatile("s_waitcnt vmcnt(28)" ::: "memory");
     if (N == 32) asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
     if (N == 48) asm volatile("s_waitcnt vmcnt(48)" ::: "memory");
 }
@@ -1274,7 +1276,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
                                                                        int *__restrict__ sk_count,
                                                                        const int32_t *__restrict__ rt, int64_t xrows)
 {
-    constexpr int WM = 2, WN = 2, NW = 4;
+    constexpr int NW = 4, WM = BM / 128, WN = NW / WM;                 // 256 x 256: 2 x 2 waves, 128 x 256: 1 x 4
     constexpr int WTM = BM / WM, WTN = BN / WN, TMS = WTM / 16, TNS = WTN / 16, HM = TMS / 2;
     constexpr int BNO = SWIGLU ? BN / 2 : BN;
     constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW, NL = LA + LB;
@@ -1282,10 +1284,11 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
     constexpr int NM = HM * TNS;
     constexpr int STG = 16 * (SWIGLU ? WTN / 2 : WTN) * 2;            // staging bytes per wave: 16 output rows
     constexpr int NS = WTM * (SWIGLU ? WTN / 2 : WTN) * 2 / 1024;      // output stores per wave and tile
-    static_assert(HM == 4 && TNS == 8 && NL == 16, "the schedule is written for 128x128 wave tiles");
+    static_assert(HM == 4 && ((TNS == 8 && NL == 16) || (TNS == 4 && NL == 12)),
+                  "the schedule is written for 128x128 and 128x64 wave tiles");
     constexpr int NOB = SWIGLU ? TNS / 2 : TNS;                       // output sub-tile columns per wave
-    constexpr bool WIDE = true;
-    static_assert(NS == 16 || NS == 32, "wait counts below");
+    constexpr bool WIDE = TNS == 8;
+    static_assert(NS == 8 || NS == 16 || NS == 32, "wait counts below");
     using frag = typename Mfma<T>::frag;
 
     extern __shared__ __attribute__((aligned(16))) char smem[];      // two stages, then NW staging regions
@@ -1336,7 +1339,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
     for (int q = 0; q < NL; ++q) OPMX_ISSUE1(0, 0, q);
 #pragma unroll
     for (int q = 0; q < NL; ++q) OPMX_ISSUE1(1, 1, q);
-    wait_vm<16>();
+    wait_vm<NL>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 #pragma unroll
@@ -1373,10 +1376,10 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
         const int nxt_tok = wave_row_index<LA * 8>(rt, nxt.row0, R, wave, lane);
 
         // k-tile 0 overwrites the accumulators.  When k-tile 1 is known to have landed, the NS
-        // stores of the previous tile and the 16 loads of this step may still be outstanding.
-        OPMX_ITERX(2, b, true, true, true, 16 + NS);
+        // stores of the previous tile and the NL loads of this step may still be outstanding.
+        OPMX_ITERX(2, b, true, true, true, NL + NS);
         b ^= 1;
-        for (int kt = 1; kt + 2 < nk; ++kt, b ^= 1) OPMX_ITERX(kt + 2, b, true, true, false, 16);
+        for (int kt = 1; kt + 2 < nk; ++kt, b ^= 1) OPMX_ITERX(kt + 2, b, true, true, false, NL);
         // all loads of this tile are issued: retarget the load state, then stream on
         rx = x_descriptor(X, nxt.row0, nxt.rows, K, rt, xrows);
         rw = raw_descriptor(W + static_cast<int64_t>(nxt.e) * N * K);
@@ -1385,9 +1388,9 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
         const int64_t nw0 = static_cast<int64_t>(cur_n) * BNO + wn * (SWIGLU ? WTN / 2 : WTN);   // first output column of this wave
         T bg[NOB][4], bu[NOB][4];          // bias of this lane's columns, requested ahead of the last loads
         if (BIAS) load_bias_regs<T, NOB, SWIGLU>(Bias + static_cast<int64_t>(cur.e) * N, ncols, nw0, lane, bg, bu);
-        OPMX_ITERX(0, b, true, true, false, 16);
+        OPMX_ITERX(0, b, true, true, false, NL);
         b ^= 1;
-        OPMX_ITERX(1, b, true, true, false, 16);
+        OPMX_ITERX(1, b, true, true, false, NL);
         b ^= 1;
         // let the last MFMAs retire; re-define the accumulators behind the wait (see
         // gemm_tiled_dlds_kernel)
@@ -1517,8 +1520,15 @@ int tiled_dlds_launch(const void *X, const int64_t *off, const void *W, const vo
     } else if (K / BK > 128) {
         persist = false;
     }
-    if constexpr (BM == 256) if (persist) {
-        const int smem_p = smem + 4 * 16 * (sw ? BN / 4 : BN / 2) * 2;       // + the four staging regions
+    {
+        // 128 x 256 tiles: the persistent form pays while a tile is short (its fixed cost of about
+        // 8 us outside the k loop is then a tenth of the tile and more)
+        if constexpr (BM == 128)
+            if (option(kOptPersist) < 0 && K / BK > 128) persist = false;
+    }
+    if (persist) {
+        constexpr int WTN_ = BN / (4 / (BM / 128));                          // columns of a wave tile
+        const int smem_p = smem + 4 * 16 * (sw ? WTN_ / 2 : WTN_) * 2;       // + the four staging regions
         static std::atomic<uint64_t> attr_p[4];
         const bool hb = B != nullptr;
         using kernel_t = void (*)(const T *, const int64_t *, const T *, const T *, int, int64_t, int64_t, int64_t, T *, int,

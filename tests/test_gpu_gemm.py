@@ -170,12 +170,13 @@ def test_expert_grouped_tile_order(variant):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_persistent_kernel_streams_tiles(dtype):
-    """The persistent form of the 256x256 kernel (16 column tiles, K >= 256): fewer tiles than
-    workgroups, then 27 row tiles x 16 = 432 tiles so that workgroups walk on to a second tile
-    (ragged row tiles, bias, SwiGLU with 16 column tiles of 128), K = 256 being the shortest
-    stream it takes; the one-tile-per-workgroup form must give the same bits."""
-    env = {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": "0", "OPMX_MOE_GEMM_STREAMK": "0"}
+@pytest.mark.parametrize("variant", ["0", "3"])
+def test_persistent_kernel_streams_tiles(dtype, variant):
+    """The persistent form of the 256x256 and of the 128x256 kernel (16 column tiles, K >= 256): fewer
+    tiles than workgroups, then 27 (128-row tiles: 50) row tiles x 16 so that workgroups walk on to a
+    second tile (ragged row tiles, bias, SwiGLU with 16 column tiles of 128), K = 256 being the
+    shortest stream it takes; the one-tile-per-workgroup form must give the same bits."""
+    env = {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": variant, "OPMX_MOE_GEMM_STREAMK": "0"}
     sizes = [1500, 0, 700, 33, 1281, 256, 5, 1300, 1024, 300]
     run_case("column", [300, 77, 129], 256, 4096, dtype, True, env)
     for K, bias, swiglu in ((256, False, False), (320, True, False), (512, True, True), (1024, False, True)):
@@ -185,6 +186,10 @@ def test_persistent_kernel_streams_tiles(dtype):
     # row-partition order (11 column tiles), several tiles per workgroup, uneven XCD shares (27 row tiles)
     a = run_case("column", sizes, 256, 2816, dtype, True, env)
     b = run_case("column", sizes, 256, 2816, dtype, True, dict(env, OPMX_MOE_GEMM_PERSIST="0"))
+    assert torch.equal(a, b)
+    # a long K, where the persistent form is taken only on request
+    a = run_case("row", sizes, 8192, 512, dtype, False, dict(env, OPMX_MOE_GEMM_PERSIST="1"))
+    b = run_case("row", sizes, 8192, 512, dtype, False, dict(env, OPMX_MOE_GEMM_PERSIST="0"))
     assert torch.equal(a, b)
     # with the tail of the last round split over k by the second launch
     run_case("row", sizes, 1024, 4096, dtype, True, dict(env, OPMX_MOE_GEMM_STREAMK="2"))
