@@ -72,7 +72,8 @@ struct RowGather {
     const int32_t *index = nullptr;
     int64_t x_rows = 0;
 };
-// The row of X that GEMM row r reads, clamped into X (a corrupt index cannot leave the tensor).
+// The row of X that GEMM row r reads, clamped into X (a corrupt index cannot leave the tensor; the
+// direct-to-LDS kernels clamp the same way where they turn the index into an offset).
 __device__ __forceinline__ int64_t gathered_row(const int32_t *__restrict__ index, int64_t x_rows, int64_t r)
 {
     const int64_t t = index[r];

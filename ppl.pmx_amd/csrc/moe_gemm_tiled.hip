@@ -779,8 +779,8 @@ constexpr uint32_t kPastEveryX = 0x80000000u;   // a byte offset no gathered X r
 // MFMA kernels against a power limit.  With SWIGLU a wave's WTN W-rows are WTN/2 gate rows
 // followed by the WTN/2 up rows of the same output columns.
 template <int LA, int LB, int WTN, bool SWIGLU>
-__device__ __forceinline__ void tile_sources(int rows, bool gather, int tokv, int64_t n0, int64_t K, int64_t N,
-                                             int64_t ncols, int wave, int lane, uint32_t (&a_src)[LA],
+__device__ __forceinline__ void tile_sources(int rows, bool gather, int tokv, int64_t xrows, int64_t n0, int64_t K,
+                                             int64_t N, int64_t ncols, int wave, int lane, uint32_t (&a_src)[LA],
                                              uint32_t (&b_src)[LB])
 {
     const int lrow8 = lane >> 3, slot = lane & 7;
@@ -793,8 +793,10 @@ __device__ __forceinline__ void tile_sources(int rows, bool gather, int tokv, in
         } else {
             // Through the row index (RowGather): offsets count from X itself.  Lane l of the wave
             // holds the index of the wave's l-th row (wave_row_index); each lane fetches the one of
-            // its row by a cross-lane read.  Rows the tile lacks get an offset past every X.
-            const int tok = __shfl(tokv, i * 8 + lrow8, 64);
+            // its row by a cross-lane read and clamps it into X, like gathered_row(): a corrupt index
+            // reads some row of X, never past it.  Rows the tile lacks get an offset past every X.
+            const int raw = __shfl(tokv, i * 8 + lrow8, 64), last = static_cast<int>(xrows) - 1;
+            const int tok = raw < 0 ? 0 : (raw > last ? last : raw);
             a_src[i] = row < rows ? static_cast<uint32_t>((static_cast<int64_t>(tok) * K + c * 8) * 2) : kPastEveryX;
         }
     }
@@ -817,7 +819,8 @@ __device__ __forceinline__ void tile_sources(int rows, bool gather, int tokv, in
 
 // Row index (RowGather) of the l-th X row that wave `wave` loads for the tile starting at row0
 // (a wave loads RW = BM / 4 consecutive tile rows), in lane l; 0 without an index.  One load per
-// lane, issued well ahead of tile_sources, which reads it across lanes.
+// lane, issued well ahead of tile_sources, which reads it across lanes and clamps it into X (the
+// value is left as loaded here: arithmetic on it would wait for the load here).
 template <int RW>
 __device__ __forceinline__ int wave_row_index(const int32_t *__restrict__ rt, int64_t row0, int64_t R, int wave, int lane)
 {
@@ -991,8 +994,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_kernel(const T *__restric
     const __amdgpu_buffer_rsrc_t rw = raw_descriptor(W + static_cast<int64_t>(mt.e) * N * K);
 
     uint32_t a_src[LA], b_src[LB];     // byte offsets from the tile's X / W base at k = 0
-    tile_sources<LA, LB, WTN, SWIGLU>(mt.rows, rt != nullptr, wave_row_index<LA * 8>(rt, mt.row0, R, wave, lane), n0, K, N,
-                                      ncols, wave, lane, a_src, b_src);
+    tile_sources<LA, LB, WTN, SWIGLU>(mt.rows, rt != nullptr, wave_row_index<LA * 8>(rt, mt.row0, R, wave, lane), xrows, n0,
+                                      K, N, ncols, wave, lane, a_src, b_src);
     const int a_lds = wave * LA * 1024, b_lds = BM * ROWB + wave * LB * 1024;   // wave-uniform
 
     float4_t acc[TNS][TMS];
@@ -1321,7 +1324,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
     __amdgpu_buffer_rsrc_t rx = x_descriptor(X, cur.row0, cur.rows, K, rt, xrows);
     __amdgpu_buffer_rsrc_t rw = raw_descriptor(W + static_cast<int64_t>(cur.e) * N * K);
     uint32_t a_src[LA], b_src[LB];
-    tile_sources<LA, LB, WTN, SWIGLU>(cur.rows, rt != nullptr, wave_row_index<LA * 8>(rt, cur.row0, R, wave, lane),
+    tile_sources<LA, LB, WTN, SWIGLU>(cur.rows, rt != nullptr, wave_row_index<LA * 8>(rt, cur.row0, R, wave, lane), xrows,
                                       static_cast<int64_t>(cur_n) * BNO, K, N, ncols, wave, lane, a_src, b_src);
     const int a_lds = wave * LA * 1024, b_lds = BM * ROWB + wave * LB * 1024;
     char *stg = smem + 2 * STAGE + wave * STG;
@@ -1383,8 +1386,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_dlds_persist_kernel(const T *_
         // all loads of this tile are issued: retarget the load state, then stream on
         rx = x_descriptor(X, nxt.row0, nxt.rows, K, rt, xrows);
         rw = raw_descriptor(W + static_cast<int64_t>(nxt.e) * N * K);
-        tile_sources<LA, LB, WTN, SWIGLU>(nxt.rows, rt != nullptr, nxt_tok, static_cast<int64_t>(nxt_n) * BNO, K, N, ncols, wave,
-                                          lane, a_src, b_src);
+        tile_sources<LA, LB, WTN, SWIGLU>(nxt.rows, rt != nullptr, nxt_tok, xrows, static_cast<int64_t>(nxt_n) * BNO, K, N, ncols,
+                                          wave, lane, a_src, b_src);
         const int64_t nw0 = static_cast<int64_t>(cur_n) * BNO + wn * (SWIGLU ? WTN / 2 : WTN);   // first output column of this wave
         T bg[NOB][4], bu[NOB][4];          // bias of this lane's columns, requested ahead of the last loads
         if (BIAS) load_bias_regs<T, NOB, SWIGLU>(Bias + static_cast<int64_t>(cur.e) * N, ncols, nw0, lane, bg, bu);

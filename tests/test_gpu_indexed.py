@@ -230,6 +230,31 @@ def test_indexed_rejects_bad_arguments():
     y = OPMX.moe_column_parallel_linear_indexed(X, bad, off, W, None, 2, 64, 32)
     torch.cuda.synchronize()
     assert bool(torch.isfinite(y.float()).all())
+    # ... in every kernel family, to the same rows: an index below 0 reads row 0, one past the end the last row
+    from torch_function import _lib
+    T, K, N, R = 96, 128, 256, 672          # seven rows per token
+    g = torch.Generator().manual_seed(3)
+    Xb = torch.randn(T, K, generator=g).half().to(d)
+    Wb = (torch.randn(2, N, K, generator=g) * 0.05).half().to(d)
+    offb = torch.tensor([0, 300, R], device=d)
+    idx = torch.randint(-50, T + 50, (R,), generator=g, dtype=torch.int32).to(d)
+    want = None
+    for env in ({"OPMX_MOE_GEMM": "generic"}, {"OPMX_MOE_GEMM": "stream"},
+                {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": "0"},
+                {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": "0", "OPMX_MOE_GEMM_PERSIST": "0"},
+                {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": "2"},
+                {"OPMX_MOE_GEMM": "tiled", "OPMX_MOE_GEMM_TILED_VARIANT": "3"}):
+        for key, val in env.items():
+            _lib.set_option(key, val)
+        try:
+            got = OPMX.moe_column_parallel_linear_indexed(Xb, idx, offb, Wb, None, 2, K, N)
+            if want is None:
+                want = OPMX.moe_column_parallel_linear_indexed(Xb, idx.clamp(0, T - 1), offb, Wb, None, 2, K, N)
+            torch.cuda.synchronize()
+        finally:
+            for key in env:
+                _lib.set_option(key, None)
+        assert float((got.float() - want.float()).abs().max()) <= 2e-2, env
 
 
 def test_indexed_gemm_on_an_empty_batch():
