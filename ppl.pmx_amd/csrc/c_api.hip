@@ -22,7 +22,7 @@ constexpr int64_t kStreamMaxRowsPerExpert = 64;
 const char *const kOptionNames[kNumOptions] = {"OPMX_MOE_GEMM", "OPMX_MOE_GEMM_TILED_VARIANT",
                                                "OPMX_MOE_GEMM_STREAM_VARIANT", "OPMX_MOE_GEMM_GNX",
                                                "OPMX_MOE_GEMM_STREAMK", "OPMX_MOE_GEMM_PERSIST",
-                                               "OPMX_MOE_ROUTE_INDEX_TOKENS"};
+                                               "OPMX_MOE_ROUTE_INDEX_TOKENS", "OPMX_MOE_GEMM_F32_VARIANT"};
 
 // Kernel family names accepted for OPMX_MOE_GEMM in the environment.
 int parse_option(int id, const char *v)

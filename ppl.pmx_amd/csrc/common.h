@@ -83,6 +83,8 @@ enum Option {
     kOptPersist,         // OPMX_MOE_GEMM_PERSIST: 0 never the persistent form, 1 whenever possible
     kOptRouteIndexTokens,  // OPMX_MOE_ROUTE_INDEX_TOKENS: up to how many tokens (0 ... 64) the index form of router
                            // gate + MoeSelect runs as one launch of one block
+    kOptF32Variant,        // OPMX_MOE_GEMM_F32_VARIANT: few rows per expert, fp32: 0 the 128-column tile form, 1 the form
+                           // whose waves split K
     kNumOptions
 };
 int option(Option o);

@@ -109,7 +109,7 @@ def test_tuning_knobs(lib):
     assert lib.opmx_moe_set_option(b"OPMX_MOE_GEMM", 2) == 0
     assert lib.opmx_moe_set_option(b"OPMX_MOE_GEMM", -1) == 0          # back to automatic
     for name in (b"OPMX_MOE_GEMM_TILED_VARIANT", b"OPMX_MOE_GEMM_STREAM_VARIANT", b"OPMX_MOE_GEMM_GNX",
-                 b"OPMX_MOE_GEMM_STREAMK", b"OPMX_MOE_GEMM_PERSIST", b"OPMX_MOE_ROUTE_INDEX_TOKENS"):
+                 b"OPMX_MOE_GEMM_STREAMK", b"OPMX_MOE_GEMM_PERSIST", b"OPMX_MOE_ROUTE_INDEX_TOKENS", b"OPMX_MOE_GEMM_F32_VARIANT"):
         assert lib.opmx_moe_set_option(name, -1) == 0
     assert lib.opmx_moe_set_option(b"OPMX_NO_SUCH_KNOB", 1) == -1
     assert lib.opmx_moe_set_option(None, 1) == -1

@@ -83,20 +83,27 @@ def test_tiny_config_fp32_shapes():
 
 @pytest.mark.parametrize("swiglu", [False, True])
 def test_fp32_matrix_unit_kernel(swiglu):
-    """fp32 tensors with K a multiple of 4 go to the fp32 MFMA kernel: 32-row tiles (few rows per expert)
-    and 128-row tiles, ragged / empty / one-row experts, K that is no multiple of the 32-wide k-tile,
-    N that is no multiple of the 128-row W tile, bias; against the float64 oracle, and close to the
-    shape-agnostic kernel (both accumulate in fp32, in different orders)."""
+    """fp32 tensors with K a multiple of 4 go to the fp32 MFMA kernels: 32-row tiles whose waves split K
+    (few rows per expert, or few tiles), 32- and 128-row tiles of 128 columns; ragged / empty / one-row
+    experts, K that is no multiple of the 32-wide k-tile, N that is no multiple of the W tile, bias;
+    against the float64 oracle, and close to the shape-agnostic kernel (both accumulate in fp32, in
+    different orders)."""
     few = [5, 0, 17, 1, 0, 31, 3, 38]
     many = [300, 0, 129, 1, 256, 77, 0, 513]
-    for sizes in (few, many):
-        for kind, K, N, bias in (("column", 128, 512, False), ("row", 100, 72, True), ("column", 36, 200, True),
-                                 ("row", 1024, 130, False), ("column", 4, 8, True)):
-            if swiglu and (kind == "row" or N % 2):
-                continue
-            a = run_case(kind, sizes, K, N, torch.float32, bias, swiglu=swiglu)
-            b = run_case(kind, sizes, K, N, torch.float32, bias, {"OPMX_MOE_GEMM": "generic"}, swiglu=swiglu)
-            assert float((a - b).abs().max()) <= 1e-4 * max(1.0, float(b.abs().max()))
+    # the library's own choice, the 128-column tile forms (32- or 128-row tiles) and the form whose waves split K
+    for variant in (None, "0", "1"):
+        env = {} if variant is None else {"OPMX_MOE_GEMM_F32_VARIANT": variant}
+        for sizes in (few, many):
+            for kind, K, N, bias in (("column", 128, 512, False), ("row", 100, 72, True), ("column", 36, 200, True),
+                                     ("row", 1024, 130, False), ("column", 4, 8, True), ("row", 2816, 96, True)):
+                if swiglu and (kind == "row" or N % 2):
+                    continue
+                a = run_case(kind, sizes, K, N, torch.float32, bias, env, swiglu=swiglu)
+                if variant is None:
+                    b = run_case(kind, sizes, K, N, torch.float32, bias, {"OPMX_MOE_GEMM": "generic"}, swiglu=swiglu)
+                    assert float((a - b).abs().max()) <= 1e-4 * max(1.0, float(b.abs().max()))
+        y = run_case("column", [9, 0, 20], 256, 64, torch.float32, True, env, off=torch.tensor([2, 11, 11, 31]), R=40, swiglu=swiglu)
+        assert float(y[:2].abs().max()) == 0.0 and float(y[31:].abs().max()) == 0.0
     # rows that belong to no expert stay zero; K % 4 != 0 falls back to the shape-agnostic kernel
     off = torch.tensor([3, 40, 40, 100], dtype=torch.int64)
     y = run_case("column", [37, 0, 60], 64, 96, torch.float32, True, off=off, R=110, swiglu=swiglu)

@@ -185,6 +185,8 @@ def test_indexed_generic_kernel(dtype, swiglu):
 @pytest.mark.parametrize("swiglu", [False, True])
 def test_indexed_fp32_matrix_unit_kernel(swiglu):
     indexed_case(RAGGED8, 64, 128, 96, torch.float32, True, swiglu=swiglu)         # 32-row tiles
+    indexed_case(RAGGED8, 64, 512, 96, torch.float32, True, {"OPMX_MOE_GEMM_F32_VARIANT": "0"}, swiglu=swiglu)
+    indexed_case(RAGGED8, 64, 512, 96, torch.float32, True, {"OPMX_MOE_GEMM_F32_VARIANT": "1"}, swiglu=swiglu)   # waves split K
     indexed_case(BIG8, 2560, 100, 256, torch.float32, False, swiglu=swiglu)        # 128-row tiles, ragged K tile
 
 
