@@ -86,6 +86,8 @@ const char *opmx_status_string(int status);
  *   "OPMX_MOE_GEMM_PERSIST"        0 never the persistent form, 1 whenever its conditions hold
  *   "OPMX_MOE_ROUTE_INDEX_TOKENS"  up to how many tokens (0 ... 64, then also up to 64 experts)
  *                                  opmx_moe_route_select_index runs as one launch of one block
+ *   "OPMX_MOE_GEMM_F32_VARIANT"    float32 grouped GEMM: 0 the 128-column tile forms only, 1 always the
+ *                                  32-row tiles whose waves split K
  * Returns OPMX_ERR_BAD_ARGUMENT for an unknown name. */
 int opmx_moe_set_option(const char *name, int value);
 
