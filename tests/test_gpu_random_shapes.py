@@ -53,6 +53,28 @@ def test_grouped_gemm_random(seed):
     run_case(kind, sizes, K, N, dtype, bias, None, seed=seed)      # automatic selection
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_grouped_gemm_random_fp32(seed):
+    """float32 tensors: the library's own choice among the fp32 matrix-unit kernels, each of their forms forced
+    (128-column tiles; 32-row tiles whose waves split K), and the shape-agnostic kernel, K any multiple of 4."""
+    rng = random.Random(3000 + seed)
+    E = rng.choice([1, 2, 3, 8, 8, 16, 31, 64, 100])
+    style = rng.choice(["sparse", "even", "skewed", "ragged"])
+    sizes = draw_sizes(rng, E, style)
+    if E >= 16:
+        sizes = [min(s, 150) for s in sizes]          # keep the float64 oracle quick
+    if sum(sizes) == 0:
+        sizes[rng.randrange(E)] = 5
+    K = rng.choice([32, 64, 128, 256, 1024]) if rng.random() < 0.5 else 4 * rng.randint(1, 200)
+    N = rng.choice([32, 64, 128, 256]) if rng.random() < 0.5 else rng.randint(1, 300)
+    bias = rng.random() < 0.5
+    kind = rng.choice(["column", "row"])
+    for env in (None, {"OPMX_MOE_GEMM_F32_VARIANT": "0"}, {"OPMX_MOE_GEMM_F32_VARIANT": "1"}, {"OPMX_MOE_GEMM": "generic"}):
+        run_case(kind, sizes, K, N, torch.float32, bias, env, seed=seed)
+        if N % 2 == 0:
+            run_case("column", sizes, K, N, torch.float32, bias, env, swiglu=True, seed=seed)
+
+
 @pytest.mark.parametrize("seed", range(40))
 def test_select_reduce_random(seed):
     rng = random.Random(5000 + seed)
