@@ -208,7 +208,7 @@ int opmx_moe_column_parallel_linear(const void *X, const int64_t *expert_offset,
  * [R] int32 with values in [0, X_rows) -- the row_token output of opmx_moe_select_index.  Equals
  * opmx_moe_column_parallel_linear on X_expand_permute bit for bit (the reference gathers first,
  * torch_function/MoeSelect.py:45-47, then multiplies, MoeColumnParallelLinear.py:58-67).
- * fp16 / bf16 kernels need X_rows * K * 2 < 2^31 (else the fp32-style fallback kernel runs). */
+ * fp16 / bf16 kernels need X_rows * K * 2 < 2^31 (else the shape-agnostic fallback kernel runs). */
 int opmx_moe_column_parallel_linear_indexed(const void *X, int64_t X_rows, const int32_t *row_index,
                                             const int64_t *expert_offset, const void *W, const void *B, int E,
                                             int64_t R, int64_t K, int64_t N, int dtype, int epilogue,
