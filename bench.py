@@ -19,8 +19,9 @@ already resident in HBM.  Prints ONE JSON line:
   hip_graph_replay     the same steps replayed from one captured HIP graph (launch cost of the
                        six operators taken off the host)
   per_op_us            mean duration of each operator (separate untimed pass)
-  device_ceilings      streaming-read GB/s and MFMA TFLOP/s (random fp16 operands) this
-                       device sustains, from the probe ppl.pmx_amd/lib/opmx_device_ceilings
+  device_ceilings      streaming-read GB/s, MFMA TFLOP/s (random fp16 operands) and the GB/s
+                       per CU at which tile operands reach LDS that this device sustains,
+                       from the probe ppl.pmx_amd/lib/opmx_device_ceilings
   vendor_dense_gemm_same_flops_TFLOPs
                        MFMA-bound workloads: the vendor library's dense GEMM with the flop
                        count of the gate/up launch (no expert grouping), context only

@@ -1,6 +1,11 @@
 // Device-ceiling probe for MI355X: what this GPU sustains for (a) a pure streaming
 // read of a weight-sized buffer and (b, c) MFMA loops (32x32x16 and 16x16x32) on random fp16
-// operands, register-fed and LDS-fed.  These are the practical ceilings the grouped-GEMM
+// operands, register-fed and LDS-fed, and (d) what one CU pulls into LDS in the tile kernels'
+// operand shape (two 256-row x 128-byte k-tiles per step, rows 2*K bytes apart, fetched with
+// buffer_load ... lds and nothing else going on): once with every workgroup re-reading tiles
+// that stay in L2, once as 32 workgroups per XCD walk K as an 8 x 4 block of output tiles
+// does (each X tile shared by 4, each W tile by 8, all of it new to the L2 at every step).
+// These are the practical ceilings the grouped-GEMM
 // kernels are compared with in addition to the vendor peaks (8 TB/s, 2.5 PFLOP/s):
 // the engine clock drops under dense MFMA load with toggling operands, so the vendor
 // MFMA peak is not reachable by any kernel on real data.
@@ -121,6 +126,46 @@ __global__ __launch_bounds__(512) void mfma16_kernel(const _Float16 *__restrict_
     out[blockIdx.x * blockDim.x + tid] = s;
 }
 
+// ---- (d) operand pull of a 256x256 output tile: per step eight 1 KiB wave loads per wave
+// (four of the X tile, four of the W tile) straight into LDS, the next step issued while one
+// is in flight.  resident: every workgroup re-reads one k-tile of its own.
+#define LPTR(p) ((void __attribute__((address_space(3))) *)(p))
+__global__ __launch_bounds__(512) void pull_kernel(const char *xbase, const char *wbase, uint32_t ld, int ktiles,
+                                                   int steps, bool resident, unsigned *out)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;   // workgroups go round the XCDs
+    const size_t tile = 256 * static_cast<size_t>(ld);
+    const char *xp = xbase + (resident ? blockIdx.x & 63 : xcd * 8 + (slot >> 2)) * tile;
+    const char *wp = wbase + (resident ? blockIdx.x & 63 : xcd * 4 + (slot & 3)) * tile;
+    auto descriptor = [](const char *base) {
+        const uint64_t b = reinterpret_cast<uint64_t>(base);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(b));
+        const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(b >> 32));
+        return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>((static_cast<uint64_t>(hi) << 32) | lo),
+                                                 0, static_cast<int>(0xFFFFFFFFu), 0x00020000);
+    };
+    const __amdgpu_buffer_rsrc_t xr = descriptor(xp), wr = descriptor(wp);
+    uint32_t voff[4];
+    for (int i = 0; i < 4; ++i) voff[i] = (8 * (wave * 4 + i) + (lane >> 3)) * ld + (lane & 7) * 16;
+    int kt = 0;
+    for (int s = 0; s < steps; ++s) {
+        const int soff = resident ? (blockIdx.x >> 6) * 128 : kt * 128;
+        char *buf = smem + (s & 1) * 65536 + wave * 8192;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(xr, LPTR(buf + i * 1024), 16, voff[i], soff, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(wr, LPTR(buf + 4096 + i * 1024), 16, voff[i], soff, 0, 0);
+        }
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        if (++kt == ktiles) kt = 0;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (reinterpret_cast<unsigned *>(smem)[tid] == 0x12345678u) out[0] = 1;
+}
+
 static float best_ms(hipEvent_t e0, hipEvent_t e1, int reps, void (*launch)(void *), void *ctx)
 {
     float best = 1e30f;
@@ -137,6 +182,7 @@ static float best_ms(hipEvent_t e0, hipEvent_t e1, int reps, void (*launch)(void
 }
 
 struct ReadCtx { const u32x4 *src; size_t n16; unsigned *out; int blocks; bool nt; };
+struct PullCtx { const char *x, *w; uint32_t ld; int ktiles, steps; bool resident; unsigned *out; };
 struct MfmaCtx { const _Float16 *src; float *out; int iters; bool lds; bool m16; };
 
 int main()
@@ -202,10 +248,30 @@ int main()
     const double mfma16_reg = flops16 / best_ms(e0, e1, 5, mfma_launch, &mc) / 1e9;
     mc.lds = true;
     const double mfma16_lds = flops16 / best_ms(e0, e1, 5, mfma_launch, &mc) / 1e9;
+    // (d): 64 X tiles and 32 W tiles of 256 rows x K = 14336 fp16 (the down projection's K)
+    const uint32_t pull_ld = 14336 * 2;
+    const size_t pull_tile = 256 * static_cast<size_t>(pull_ld);
+    char *px, *pw;
+    CHECK(hipMalloc(&px, 64 * pull_tile));
+    CHECK(hipMalloc(&pw, 64 * pull_tile));
+    CHECK(hipMemset(px, 1, 64 * pull_tile));
+    CHECK(hipMemset(pw, 2, 64 * pull_tile));
+    CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(pull_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              131072));
+    PullCtx pc{px, pw, pull_ld, static_cast<int>(pull_ld / 128), 4000, true, flag};
+    auto pull_launch = [](void *c) {
+        PullCtx *p = static_cast<PullCtx *>(c);
+        pull_kernel<<<256, 512, 131072>>>(p->x, p->w, p->ld, p->ktiles, p->steps, p->resident, p->out);
+    };
+    const double pull_resident = 65536.0 * pc.steps / best_ms(e0, e1, 4, pull_launch, &pc) / 1e6;
+    pc.resident = false;
+    const double pull_streamed = 65536.0 * pc.steps / best_ms(e0, e1, 4, pull_launch, &pc) / 1e6;
     CHECK(hipGetLastError());
     printf("{\"hbm_read_GBs\": %.0f, \"hbm_read_nontemporal_GBs\": %.0f, "
            "\"mfma_f16_register_fed_TFLOPs\": %.0f, \"mfma_f16_lds_fed_TFLOPs\": %.0f, "
-           "\"mfma_f16_16x16x32_register_fed_TFLOPs\": %.0f, \"mfma_f16_16x16x32_lds_fed_TFLOPs\": %.0f}\n",
-           read_plain, read_nt, mfma_reg, mfma_lds, mfma16_reg, mfma16_lds);
+           "\"mfma_f16_16x16x32_register_fed_TFLOPs\": %.0f, \"mfma_f16_16x16x32_lds_fed_TFLOPs\": %.0f, "
+           "\"tile_operands_to_lds_L2_resident_GBs_per_CU\": %.1f, "
+           "\"tile_operands_to_lds_streamed_8x4_per_XCD_GBs_per_CU\": %.1f}\n",
+           read_plain, read_nt, mfma_reg, mfma_lds, mfma16_reg, mfma16_lds, pull_resident, pull_streamed);
     return 0;
 }
