@@ -94,3 +94,8 @@ def test_bench_json_line():
     assert abs(d["value"] - 8 / (d["ms_per_step"] * 1e-3)) / d["value"] < 1e-3
     c = d["cpu_baseline"]
     assert c["kind"] == "port" and c["cores"] >= 1 and c["value"] > 0 and "sample" in c
+    # what the device sustains, from the probe beside the library: operands that stay in L2 reach LDS
+    # faster than operands streamed in the tile kernels' pattern, and both are real rates
+    dc = d["device_ceilings"]
+    assert dc["hbm_read_nontemporal_GBs"] > 1000 and dc["mfma_f16_16x16x32_lds_fed_TFLOPs"] > 100
+    assert dc["tile_operands_to_lds_L2_resident_GBs_per_CU"] > dc["tile_operands_to_lds_streamed_8x4_per_XCD_GBs_per_CU"] > 5
